@@ -2,8 +2,10 @@
 // whose queries see a SPAN of the keys: the last `window` keys (window 0: all earlier keys) plus the
 // first `keep_first` keys of the sequence, which are never dropped.  Query at position i sees key j when
 //     j <= i  and  (window == 0  or  i - j < window  or  j < keep_first).
-// `sink` adds one term exp(0) to the softmax's denominator that has no value:
-//     p_j = exp(s_j) / (sink + sum_j exp(s_j)).
+// `sink` adds one term to the softmax's denominator that has no value, exp(0) or, with `sinks` (one float32
+// per head, a learned number), exp(sinks[h]):
+//     p_j = exp(s_j) / (exp(sink_h) + sum_j exp(s_j)).
+// `softcap` c > 0 bounds the scaled score before the softmax: s <- c tanh(s / c).  The sink is neither scaled nor capped.
 // `gate` (nullable): the result is multiplied element by element with sigmoid(gate[t, h * dv + d]).
 // Scores, the running softmax and the sums are float32.
 //
@@ -41,7 +43,7 @@ attn_span_generic_kernel(const T* __restrict__ q, int q_stride, T* __restrict__ 
                          const int* __restrict__ block_tables, int bt_stride,
                          const int* __restrict__ token_req, const int* __restrict__ positions,
                          int nh, int nkvh, int dk, int dv, int page_size, float scale, int window, int keep_first,
-                         int sink) {
+                         int sink, const float* __restrict__ sinks, float softcap) {
     __shared__ float qs[kSpanMaxDim];
     __shared__ float ps[64];
     __shared__ long long vrow[64];
@@ -76,6 +78,7 @@ attn_span_generic_kernel(const T* __restrict__ q, int q_stride, T* __restrict__ 
             float dot = 0.f;
             for (int d = 0; d < dk; ++d) dot += qs[d] * to_f32(kp[d]);
             s = dot * scale;
+            if (softcap > 0.f) s = softcap * tanhf(s / softcap);
         }
         const float m_new = fmaxf(m, wave_max(s));       // lane 0 of every chunk is valid: m_new is finite
         const float p = valid ? expf(s - m_new) : 0.f;
@@ -98,10 +101,11 @@ attn_span_generic_kernel(const T* __restrict__ q, int q_stride, T* __restrict__ 
             }
         }
     }
-    if (sink) {                                           // the term exp(0 - m) joins the denominator
-        const float m_new = fmaxf(m, 0.f);
+    if (sink) {                                           // the term exp(sink - m) joins the denominator
+        const float sv = sinks ? sinks[h] : 0.f;
+        const float m_new = fmaxf(m, sv);
         const float corr = expf(m - m_new);
-        l = l * corr + expf(-m_new);
+        l = l * corr + expf(sv - m_new);
 #pragma unroll
         for (int i = 0; i < kSpanMaxDim / 64; ++i) acc[i] *= corr;
     }
@@ -123,7 +127,7 @@ IC_EXPORT int ic_attn_span_generic(const void* q, int q_stride, void* out, int o
                                    int gate_stride, int dtype, const void* kcache, const void* vcache,
                                    const int* block_tables, int bt_stride, const int* token_req, const int* positions,
                                    int T, int nh, int nkvh, int dk, int dv, int page_size, float scale, int window,
-                                   int keep_first, int sink, hipStream_t stream) {
+                                   int keep_first, int sink, const float* sinks, float softcap, hipStream_t stream) {
     if (T <= 0) return IC_OK;
     if (nh <= 0 || nkvh <= 0 || nh % nkvh || dk <= 0 || dk > kSpanMaxDim || dv <= 0 || dv > kSpanMaxDim ||
         page_size <= 0 || window < 0 || keep_first < 0)
@@ -134,12 +138,12 @@ IC_EXPORT int ic_attn_span_generic(const void* q, int q_stride, void* out, int o
         hipLaunchKernelGGL(attn_span_generic_kernel<float>, grid, block, 0, stream, (const float*)q, q_stride, (float*)out,
                            out_stride, (const float*)gate, gate_stride, (const float*)kcache, (const float*)vcache,
                            block_tables, bt_stride, token_req, positions, nh, nkvh, dk, dv, page_size, scale, window,
-                           keep_first, sink);
+                           keep_first, sink, sinks, softcap);
     else if (dtype == IC_BF16)
         hipLaunchKernelGGL(attn_span_generic_kernel<bf16>, grid, block, 0, stream, (const bf16*)q, q_stride, (bf16*)out,
                            out_stride, (const bf16*)gate, gate_stride, (const bf16*)kcache, (const bf16*)vcache,
                            block_tables, bt_stride, token_req, positions, nh, nkvh, dk, dv, page_size, scale, window,
-                           keep_first, sink);
+                           keep_first, sink, sinks, softcap);
     else
         return IC_ERR_UNSUPPORTED;
     return ic_launch_status();
@@ -189,8 +193,8 @@ attn_span_decode_kernel(const T* __restrict__ q, int q_stride, const T* __restri
                         const int* __restrict__ block_tables, int bt_stride, const int* __restrict__ tok_list,
                         const int* __restrict__ token_req, const int* __restrict__ positions,
                         float* __restrict__ part_acc, float* __restrict__ part_ml, int nh, int nkvh, int page_size,
-                        float scale, int window, int keep_first, int nsplit, int sink,
-                        T* __restrict__ final_out, int out_stride, const T* __restrict__ gate, int gate_stride) {
+                        float scale, int window, int keep_first, int nsplit, int sink, const float* __restrict__ sinks,
+                        float softcap, T* __restrict__ final_out, int out_stride, const T* __restrict__ gate, int gate_stride) {
     constexpr int VEC = SpanVec<T>::N;
     constexpr int LPK = DK / VEC;                  // lanes per key
     constexpr int LPV = DV / VEC;                  // 16-byte pieces of a value row
@@ -214,7 +218,9 @@ attn_span_decode_kernel(const T* __restrict__ q, int q_stride, const T* __restri
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int sub = lane % LPK, grp = lane / LPK;
-    const float qscale = scale * kLog2e;           // scores in units of log 2
+    // scores in units of log 2; with a cap c the query carries scale / c and the score becomes (c log2 e) tanh(.)
+    const float qscale = softcap > 0.f ? scale / softcap : scale * kLog2e;
+    const float cap2 = softcap * kLog2e;
 
     for (int h0 = 0; h0 < g; h0 += GQ) {
         float qv[GQ][VEC], acc[GQ][NVS * VEC], m[GQ], l[GQ];
@@ -269,6 +275,7 @@ attn_span_decode_kernel(const T* __restrict__ q, int q_stride, const T* __restri
 #pragma unroll
                     for (int i = 0; i < VEC; ++i) d += qv[j][i] * kf[u][i];
                     d = group_sum<LPK>(d);                  // over the lanes that share the key (DPP steps inside a row of 16 lanes)
+                    if (softcap > 0.f) d = cap2 * tanhf(d);
                     s[u] = ok[u] ? d : -INFINITY;
                     mx = fmaxf(mx, s[u]);
                 }
@@ -333,9 +340,10 @@ attn_span_decode_kernel(const T* __restrict__ q, int q_stride, const T* __restri
             const int h = kvh * g + h0 + j;
             if (final_out) {                            // a single split: this is the result, no second pass
                 if (sink) {
-                    const float mf = fmaxf(mm, 0.f), c = __builtin_amdgcn_exp2f(mm - mf);
+                    const float sv = sinks ? sinks[h] * kLog2e : 0.f;
+                    const float mf = fmaxf(mm, sv), c = __builtin_amdgcn_exp2f(mm - mf);
                     a *= c;
-                    ll = ll * c + __builtin_amdgcn_exp2f(-mf);
+                    ll = ll * c + __builtin_amdgcn_exp2f(sv - mf);
                 }
                 float o = a / ll;
                 if (gate) o *= sigmoid_f(to_f32(gate[(size_t)t * gate_stride + (size_t)h * DV + d]));
@@ -353,13 +361,15 @@ attn_span_decode_kernel(const T* __restrict__ q, int q_stride, const T* __restri
 template <typename T>
 __global__ void attn_span_reduce_kernel(const float* __restrict__ part_acc, const float* __restrict__ part_ml,
                                         const int* __restrict__ tok_list, T* __restrict__ out, int out_stride,
-                                        const T* __restrict__ gate, int gate_stride, int nh, int dv, int nsplit, int sink) {
+                                        const T* __restrict__ gate, int gate_stride, int nh, int dv, int nsplit, int sink,
+                                        const float* __restrict__ sinks) {
     const int n = blockIdx.x / nh, h = blockIdx.x % nh;
     const int t = tok_list ? tok_list[n] : n;
     const size_t base = ((size_t)n * nh + h) * nsplit;
-    float mm = sink ? 0.f : -INFINITY;
+    const float sv = (sink && sinks) ? sinks[h] * kLog2e : 0.f;      // in units of log 2, as the partial maxima
+    float mm = sink ? sv : -INFINITY;
     for (int s = 0; s < nsplit; ++s) mm = fmaxf(mm, part_ml[(base + s) * 2]);
-    float den = sink ? __builtin_amdgcn_exp2f(-mm) : 0.f;
+    float den = sink ? __builtin_amdgcn_exp2f(sv - mm) : 0.f;
     for (int s = 0; s < nsplit; ++s) {
         const float ms = part_ml[(base + s) * 2];
         if (ms != -INFINITY) den += part_ml[(base + s) * 2 + 1] * __builtin_amdgcn_exp2f(ms - mm);
@@ -398,13 +408,14 @@ static int span_decode_launch(const void* q, int q_stride, void* out, int out_st
                               const void* kcache, const void* vcache, const int* block_tables, int bt_stride,
                               const int* tok_list, const int* token_req, const int* positions, float* part_acc,
                               float* part_ml, int n_tok, int nh, int nkvh, int page_size, float scale, int window,
-                              int keep_first, int sink, int nsplit, hipStream_t stream) {
+                              int keep_first, int sink, const float* sinks, float softcap, int nsplit, hipStream_t stream) {
     dim3 grid(nsplit, nkvh, n_tok), block(kSdThreads);
     const int g = nh / nkvh;
 #define IC_SPAN_GQ(GQ)                                                                                                          \
     hipLaunchKernelGGL((attn_span_decode_kernel<T, DK, DV, GQ>), grid, block, 0, stream, (const T*)q, q_stride, (const T*)kcache, \
                        (const T*)vcache, block_tables, bt_stride, tok_list, token_req, positions, part_acc, part_ml, nh, nkvh,   \
-                       page_size, scale, window, keep_first, nsplit, sink, nsplit == 1 ? (T*)out : (T*)nullptr, out_stride,     \
+                       page_size, scale, window, keep_first, nsplit, sink, sinks, softcap,                                       \
+                       nsplit == 1 ? (T*)out : (T*)nullptr, out_stride,                                                          \
                        (const T*)gate, gate_stride)
     if (g == 1) IC_SPAN_GQ(1);                      // query heads served per walk over the keys: no more than there are
     else if (g == 2) IC_SPAN_GQ(2);
@@ -413,7 +424,7 @@ static int span_decode_launch(const void* q, int q_stride, void* out, int out_st
     int st = ic_launch_status();
     if (st != IC_OK || nsplit == 1) return st;
     hipLaunchKernelGGL(attn_span_reduce_kernel<T>, dim3((unsigned)(n_tok * nh)), dim3(DV < 64 ? 64 : DV), 0, stream, part_acc,
-                       part_ml, tok_list, (T*)out, out_stride, (const T*)gate, gate_stride, nh, DV, nsplit, sink);
+                       part_ml, tok_list, (T*)out, out_stride, (const T*)gate, gate_stride, nh, DV, nsplit, sink, sinks);
     return ic_launch_status();
 }
 
@@ -422,12 +433,12 @@ static int span_decode_dims(int dk, int dv, const void* q, int q_stride, void* o
                             int gate_stride, const void* kcache, const void* vcache, const int* block_tables, int bt_stride,
                             const int* tok_list, const int* token_req, const int* positions, float* part_acc, float* part_ml,
                             int n_tok, int nh, int nkvh, int page_size, float scale, int window, int keep_first, int sink,
-                            int nsplit, hipStream_t stream) {
+                            const float* sinks, float softcap, int nsplit, hipStream_t stream) {
 #define IC_SPAN_DEC(K, V)                                                                                                   \
     if (dk == K && dv == V)                                                                                                 \
         return span_decode_launch<T, K, V>(q, q_stride, out, out_stride, gate, gate_stride, kcache, vcache, block_tables,   \
                                            bt_stride, tok_list, token_req, positions, part_acc, part_ml, n_tok, nh, nkvh,   \
-                                           page_size, scale, window, keep_first, sink, nsplit, stream);
+                                           page_size, scale, window, keep_first, sink, sinks, softcap, nsplit, stream);
     IC_SPAN_DEC(32, 32) IC_SPAN_DEC(32, 64) IC_SPAN_DEC(32, 128)
     IC_SPAN_DEC(64, 32) IC_SPAN_DEC(64, 64) IC_SPAN_DEC(64, 128)
     IC_SPAN_DEC(128, 32) IC_SPAN_DEC(128, 64) IC_SPAN_DEC(128, 128)
@@ -440,7 +451,8 @@ IC_EXPORT int ic_attn_span_decode(const void* q, int q_stride, void* out, int ou
                                   int dtype, const void* kcache, const void* vcache, const int* block_tables, int bt_stride,
                                   const int* tok_list, const int* token_req, const int* positions, float* part_acc,
                                   float* part_ml, int n_tok, int nh, int nkvh, int dk, int dv, int page_size, float scale,
-                                  int window, int keep_first, int sink, int nsplit, hipStream_t stream) {
+                                  int window, int keep_first, int sink, const float* sinks, float softcap, int nsplit,
+                                  hipStream_t stream) {
     if (n_tok <= 0) return IC_OK;
     if (nh <= 0 || nkvh <= 0 || nh % nkvh || page_size <= 0 || window < 0 || keep_first < 0 || nsplit < 1 || nsplit > 32)
         return IC_ERR_ARG;
@@ -450,10 +462,10 @@ IC_EXPORT int ic_attn_span_decode(const void* q, int q_stride, void* out, int ou
     if (dtype == IC_F32)
         return span_decode_dims<float>(dk, dv, q, q_stride, out, out_stride, gate, gate_stride, kcache, vcache, block_tables,
                                        bt_stride, tok_list, token_req, positions, part_acc, part_ml, n_tok, nh, nkvh, page_size,
-                                       scale, window, keep_first, sink, nsplit, stream);
+                                       scale, window, keep_first, sink, sinks, softcap, nsplit, stream);
     return span_decode_dims<bf16>(dk, dv, q, q_stride, out, out_stride, gate, gate_stride, kcache, vcache, block_tables,
                                   bt_stride, tok_list, token_req, positions, part_acc, part_ml, n_tok, nh, nkvh, page_size,
-                                  scale, window, keep_first, sink, nsplit, stream);
+                                  scale, window, keep_first, sink, sinks, softcap, nsplit, stream);
 }
 
 // =============================================================================================
@@ -489,7 +501,9 @@ attn_span_prefill_kernel(const uint16_t* __restrict__ q, int q_stride, uint16_t*
                          const uint16_t* __restrict__ gate, int gate_stride,
                          const uint16_t* __restrict__ kcache, const uint16_t* __restrict__ vcache,
                          const int* __restrict__ block_tables, int bt_stride, const int4* __restrict__ tiles,
-                         int nh, int nkvh, int page_shift, float scale_log2e, int window, int keep_first, int sink) {
+                         int nh, int nkvh, int page_shift, float scale_log2e, int window, int keep_first, int sink,
+                         const float* __restrict__ sinks, float cap_in) {
+    // cap_in > 0: a raw score s becomes tanh(s * cap_in) (cap_in = scale / cap) and scale_log2e holds cap * log2 e
     constexpr int NC = DK / 16;           // 16-wide chunks of the key size
     constexpr int ND = DV / 32;           // 32-row tiles of O^T
     constexpr int PK = DK + 8;            // padded row pitches in LDS (elements)
@@ -623,6 +637,15 @@ attn_span_prefill_kernel(const uint16_t* __restrict__ q, int q_stride, uint16_t*
                 sacc[tt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qf[c], sacc[tt], 0, 0, 0);
             }
         }
+        if (cap_in > 0.f) {                                // tanh(z) = 1 - 2 / (1 + e^(2z)): finite for every z
+#pragma unroll
+            for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const float e = __builtin_amdgcn_exp2f(sacc[tt][r] * (2.f * kLog2e * cap_in));
+                    sacc[tt][r] = 1.f - 2.f * __builtin_amdgcn_rcpf(1.f + e);
+                }
+        }
         // ---- mask: the run's bounds, the diagonal, the window and the kept first keys --------
         const bool all_seen = kb >= klo && kb + kSpKeys - 1 <= khi && kb + kSpKeys - 1 <= wave_first
                               && (window == 0 || wave_last - kb < window || kb + kSpKeys - 1 < keep_first);
@@ -698,11 +721,12 @@ attn_span_prefill_kernel(const uint16_t* __restrict__ q, int q_stride, uint16_t*
     }
 
     if (!row_ok) return;
-    if (sink) {                                            // exp(0 - m) joins the denominator
-        const float mc = (m == -INFINITY) ? 0.f : m * scale_log2e;
-        const float mf = fmaxf(mc, 0.f);
+    if (sink) {                                            // exp(sink - m) joins the denominator
+        const float sv = sinks ? sinks[h] * kLog2e : 0.f;
+        const float mc = (m == -INFINITY) ? sv : m * scale_log2e;
+        const float mf = fmaxf(mc, sv);
         const float corr = (m == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(mc - mf);
-        l = l * corr + __builtin_amdgcn_exp2f(-mf);
+        l = l * corr + __builtin_amdgcn_exp2f(sv - mf);
 #pragma unroll
         for (int i = 0; i < ND; ++i)
 #pragma unroll
@@ -740,7 +764,7 @@ IC_EXPORT int ic_attn_span_prefill_supported(int dtype, int dk, int dv) {
 IC_EXPORT int ic_attn_span_prefill(const void* q, int q_stride, void* out, int out_stride, const void* gate, int gate_stride,
                                    int dtype, const void* kcache, const void* vcache, const int* block_tables, int bt_stride,
                                    const int* tiles, int n_tiles, int nh, int nkvh, int dk, int dv, int page_size, float scale,
-                                   int window, int keep_first, int sink, hipStream_t stream) {
+                                   int window, int keep_first, int sink, const float* sinks, float softcap, hipStream_t stream) {
     if (n_tiles <= 0) return IC_OK;
     if (nh <= 0 || nkvh <= 0 || nh % nkvh || page_size <= 0 || window < 0 || keep_first < 0 || !(scale > 0.f)) return IC_ERR_ARG;
     if (!ic_attn_span_prefill_supported(dtype, dk, dv) || (page_size & (page_size - 1))) return IC_ERR_UNSUPPORTED;
@@ -751,13 +775,14 @@ IC_EXPORT int ic_attn_span_prefill(const void* q, int q_stride, void* out, int o
         return IC_ERR_ARG;
     if ((long long)n_tiles * nh > 0x7fffffffLL) return IC_ERR_ARG;
     dim3 grid((unsigned)(n_tiles * nh)), block(256);
-    const float c = scale * kLog2e;
+    const float c = softcap > 0.f ? softcap * kLog2e : scale * kLog2e;
+    const float cap_in = softcap > 0.f ? scale / softcap : 0.f;
 #define IC_SPAN_PRE(K, V)                                                                                                     \
     if (dk == K && dv == V) {                                                                                                 \
         hipLaunchKernelGGL((attn_span_prefill_kernel<K, V>), grid, block, 0, stream, (const uint16_t*)q, q_stride,            \
                            (uint16_t*)out, out_stride, (const uint16_t*)gate, gate_stride, (const uint16_t*)kcache,           \
                            (const uint16_t*)vcache, block_tables, bt_stride, (const int4*)tiles, nh, nkvh, page_shift, c,      \
-                           window, keep_first, sink);                                                                         \
+                           window, keep_first, sink, sinks, cap_in);                                                          \
         return ic_launch_status();                                                                                            \
     }
     IC_SPAN_PRE(32, 32) IC_SPAN_PRE(32, 64) IC_SPAN_PRE(32, 128)

@@ -27,6 +27,8 @@ int ic_add_rmsnorm(float* x, const void* y, int y_dtype, float alpha, const floa
 int ic_residual_add(float* x, const void* y, int y_dtype, float alpha, long long n, hipStream_t stream);
 // out[t, j] = up * silu(gate), gate = gate_up[t, j], up = gate_up[t, di + j].
 int ic_swiglu(const void* gate_up, void* out, int dtype, int T, int di, hipStream_t stream);
+// out[t, j] = g * sigmoid(alpha * g) * (u + 1), g = min(gate, limit), u = clamp(up, -limit, limit); gate_up as for ic_swiglu
+int ic_glu_clamped(const void* gate_up, void* out, int dtype, int T, int di, float limit, float alpha, hipStream_t stream);
 
 // Whole cache pages copied inside a group's planes (n_planes planes of n_pages pages of page_bytes bytes, contiguous):
 // planes[p][dst[i]] = planes[p][src[i]] for every plane p.  src, dst: device int32 [n_pairs]; no page both read and written.
@@ -80,16 +82,16 @@ int ic_activation(const void* in, void* out, int dtype, long long n, int kind, h
 // ---- attn_span.hip: keys and values of different sizes, a window plus kept first keys, a sink, an output gate --------
 // Query at position i sees key j when j <= i and (window == 0 or i - j < window or j < keep_first); sink: 1 joins the
 // softmax's denominator; gate (nullable): out *= sigmoid(gate[t, h dv + d]).
-int ic_attn_span_generic(const void* q, int q_stride, void* out, int out_stride, const void* gate, int gate_stride, int dtype, const void* kcache, const void* vcache, const int* block_tables, int bt_stride, const int* token_req, const int* positions, int T, int nh, int nkvh, int dk, int dv, int page_size, float scale, int window, int keep_first, int sink, hipStream_t stream);
+int ic_attn_span_generic(const void* q, int q_stride, void* out, int out_stride, const void* gate, int gate_stride, int dtype, const void* kcache, const void* vcache, const int* block_tables, int bt_stride, const int* token_req, const int* positions, int T, int nh, int nkvh, int dk, int dv, int page_size, float scale, int window, int keep_first, int sink, const float* sinks, float softcap, hipStream_t stream);
 
 // Single new tokens, split over the visible keys (key and value sizes 32, 64, 128; float32 or bfloat16).  tok_list (nullable): the rows that are
 // single tokens.  part_acc: float32 [n_tok, nh, nsplit, dv]; part_ml: float32 [n_tok, nh, nsplit, 2]; nsplit <= 32 (1: no second pass, no scratch).
 int ic_attn_span_decode_supported(int dtype, int dk, int dv);
 int ic_attn_span_decode_splits(int n_rows, int n_kv_heads, int max_keys, int compute_units);
-int ic_attn_span_decode(const void* q, int q_stride, void* out, int out_stride, const void* gate, int gate_stride, int dtype, const void* kcache, const void* vcache, const int* block_tables, int bt_stride, const int* tok_list, const int* token_req, const int* positions, float* part_acc, float* part_ml, int n_tok, int nh, int nkvh, int dk, int dv, int page_size, float scale, int window, int keep_first, int sink, int nsplit, hipStream_t stream);
+int ic_attn_span_decode(const void* q, int q_stride, void* out, int out_stride, const void* gate, int gate_stride, int dtype, const void* kcache, const void* vcache, const int* block_tables, int bt_stride, const int* tok_list, const int* token_req, const int* positions, float* part_acc, float* part_ml, int n_tok, int nh, int nkvh, int dk, int dv, int page_size, float scale, int window, int keep_first, int sink, const float* sinks, float softcap, int nsplit, hipStream_t stream);
 // Prompt portions on the matrix cores (bfloat16; key and value sizes 32, 64, 128; scale > 0).  tiles as for ic_attn_prefill, rows <= 128.
 int ic_attn_span_prefill_supported(int dtype, int dk, int dv);
-int ic_attn_span_prefill(const void* q, int q_stride, void* out, int out_stride, const void* gate, int gate_stride, int dtype, const void* kcache, const void* vcache, const int* block_tables, int bt_stride, const int* tiles, int n_tiles, int nh, int nkvh, int dk, int dv, int page_size, float scale, int window, int keep_first, int sink, hipStream_t stream);
+int ic_attn_span_prefill(const void* q, int q_stride, void* out, int out_stride, const void* gate, int gate_stride, int dtype, const void* kcache, const void* vcache, const int* block_tables, int bt_stride, const int* tiles, int n_tiles, int nh, int nkvh, int dk, int dv, int page_size, float scale, int window, int keep_first, int sink, const float* sinks, float softcap, hipStream_t stream);
 
 // ---- gemm.hip ---------------------------------------------------------------------------------------
 // A norm y = x * rsqrt(mean(x^2) + eps) * w between two products of M <= 16 rows can be split over them: the

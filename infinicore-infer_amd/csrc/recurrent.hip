@@ -191,14 +191,17 @@ IC_EXPORT int ic_rglru_scan(const float* gates, const float* gate_bias, const fl
 }
 
 // ---- state-space recurrence with a matrix state per head ---------------------------------------------------------
-// xbc [T, inner + 2 G N] float32 holds x (heads x P), then B (G x N), then C (G x N) of every token.  Per head h
-// with group g = h / (heads / G), dt = softplus(dt_raw + dt_bias[h]):
+// xbc [T, x_stride >= inner + 2 G N] (float32, or the step's compute dtype; in_act 1: silu on the way in) holds x
+// (heads x P), then B (G x N), then C (G x N) of every token.  Per head h with group g = h / (heads / G),
+// dt = softplus(dt_raw + dt_bias[h]):
 //     S <- exp(neg_a[h] dt) S + dt B_g x_h^T   (S is N x P),   y_h = S^T C_g + D[h] x_h.
+// Without step sizes (dt_raw null) the decay is fixed per head and every step is one: S <- neg_a[h] S + B_g x_h^T
+// (neg_a then holds the decay itself): linear attention with keys B, values x and queries C.  D null: no skip term.
 // One block per (head, request, chunk).  Thread (grp, p) keeps column p of a run of NI rows of S in registers;
 // a token's B, C and x pass through LDS, the next token's are loaded while this one is computed.
 template <typename T, int NI, bool FULL>       // FULL: every thread owns exactly NI rows (N = NI * groups): no guards, 16-byte LDS reads
 __global__ void __launch_bounds__(256)
-ssm_scan_kernel(const float* __restrict__ xbc, const T* __restrict__ dt_raw, int dt_stride,
+ssm_scan_kernel(const void* __restrict__ xbc, int x_stride, int x_f32, int in_act, const T* __restrict__ dt_raw, int dt_stride,
                 const float* __restrict__ dt_bias, const float* __restrict__ neg_a, const float* __restrict__ Dw,
                 int heads, int P, int N, int G, float* __restrict__ y, float* __restrict__ state,
                 long long state_stride, const int* __restrict__ req_start, const int* __restrict__ state_slots,
@@ -209,7 +212,7 @@ ssm_scan_kernel(const float* __restrict__ xbc, const T* __restrict__ dt_raw, int
     const int begin = req_start[r] + (mode ? ck * chunk_len : 0);
     const int end = mode ? min(req_end, begin + chunk_len) : req_end;
     if (begin >= req_end) return;
-    const int g = h / (heads / G), inner = heads * P, ch = inner + 2 * G * N;
+    const int g = h / (heads / G), inner = heads * P;
     const int ngrp = 256 / P, ni = (N + ngrp - 1) / ngrp;       // P <= 256, ni <= NI
     const int grp = tid / P, p = tid % P, n0 = grp * ni;
     const bool active = grp < ngrp;
@@ -226,36 +229,41 @@ ssm_scan_kernel(const float* __restrict__ xbc, const T* __restrict__ dt_raw, int
         const bool ok = active && i < ni && n < N;
         s[i] = !ok ? 0.f : mode == 0 ? st[n * P + p] : mode == 2 ? sc[n * P + p] : 0.f;
     }
-    const float db = dt_bias[h], na = neg_a[h], dw = Dw[h];
+    const float db = dt_bias ? dt_bias[h] : 0.f, na = neg_a[h], dw = Dw ? Dw[h] : 0.f;
+    // a token's inputs as they lie in memory: float32, or the step's compute dtype (a projection's own rows), with silu on the way in
+    auto ldx = [&](size_t i) -> float {
+        const float v = x_f32 ? reinterpret_cast<const float*>(xbc)[i] : to_f32(reinterpret_cast<const T*>(xbc)[i]);
+        return in_act ? silu_f(v) : v;
+    };
     const int off_b = inner + g * N, off_c = inner + G * N + g * N, off_x = h * P;
     auto src = [&](int e) { return e < N ? off_b + e : e < 2 * N ? off_c + (e - N) : off_x + (e - 2 * N); };
     float pre[4];
     {
-        const float* row = xbc + (size_t)begin * ch;
+        const size_t row = (size_t)begin * x_stride;
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
             const int e = tid + 256 * k;
-            if (e < bufsz) buf0[e] = row[src(e)];
+            if (e < bufsz) buf0[e] = ldx(row + src(e));
         }
     }
-    float dt_next = to_f32(dt_raw[(size_t)begin * dt_stride + h]);
+    float dt_next = dt_raw ? to_f32(dt_raw[(size_t)begin * dt_stride + h]) : 0.f;
     float a_total = 1.f;
     __syncthreads();
     for (int t = begin; t < end; ++t) {
         float* cur = ((t - begin) & 1) ? buf1 : buf0;
         float* nxt = ((t - begin) & 1) ? buf0 : buf1;
-        const float dt = softplus_f(dt_next + db);
+        const float dt = dt_raw ? softplus_f(dt_next + db) : 1.f;       // no step sizes: a fixed decay per head, steps of one
         const bool more = t + 1 < end;
         if (more) {
-            const float* row = xbc + (size_t)(t + 1) * ch;
+            const size_t row = (size_t)(t + 1) * x_stride;
 #pragma unroll
             for (int k = 0; k < 4; ++k) {
                 const int e = tid + 256 * k;
-                if (e < bufsz) pre[k] = row[src(e)];
+                if (e < bufsz) pre[k] = ldx(row + src(e));
             }
-            dt_next = to_f32(dt_raw[(size_t)(t + 1) * dt_stride + h]);
+            if (dt_raw) dt_next = to_f32(dt_raw[(size_t)(t + 1) * dt_stride + h]);
         }
-        const float da = expf(na * dt);
+        const float da = dt_raw ? expf(na * dt) : na;
         a_total *= da;
         const float* Bs = cur;
         const float* Cs = cur + N;
@@ -312,7 +320,8 @@ ssm_scan_kernel(const float* __restrict__ xbc, const T* __restrict__ dt_raw, int
 }
 
 template <typename T>
-static int ssm_launch(int ni, dim3 grid, size_t lds, hipStream_t stream, const float* xbc, const void* dt_raw, int dt_stride,
+static int ssm_launch(int ni, dim3 grid, size_t lds, hipStream_t stream, const void* xbc, int x_stride, int x_f32, int in_act,
+                      const void* dt_raw, int dt_stride,
                       const float* dt_bias, const float* neg_a, const float* Dw, int heads, int P, int N, int G, float* y,
                       float* state, long long state_stride, const int* req_start, const int* state_slots, int mode,
                       int chunk_len, int max_chunks, float* scr_s, float* scr_a) {
@@ -320,11 +329,11 @@ static int ssm_launch(int ni, dim3 grid, size_t lds, hipStream_t stream, const f
 #define IC_SSM(NI)                                                                                                      \
     do {                                                                                                                \
     if (full && ni == NI)                                                                                               \
-        hipLaunchKernelGGL((ssm_scan_kernel<T, NI, true>), grid, dim3(256), lds, stream, xbc, (const T*)dt_raw, dt_stride, \
+        hipLaunchKernelGGL((ssm_scan_kernel<T, NI, true>), grid, dim3(256), lds, stream, xbc, x_stride, x_f32, in_act, (const T*)dt_raw, dt_stride, \
                            dt_bias, neg_a, Dw, heads, P, N, G, y, state, state_stride, req_start, state_slots, mode,     \
                            chunk_len, max_chunks, scr_s, scr_a);                                                         \
     else                                                                                                                \
-        hipLaunchKernelGGL((ssm_scan_kernel<T, NI, false>), grid, dim3(256), lds, stream, xbc, (const T*)dt_raw, dt_stride, \
+        hipLaunchKernelGGL((ssm_scan_kernel<T, NI, false>), grid, dim3(256), lds, stream, xbc, x_stride, x_f32, in_act, (const T*)dt_raw, dt_stride, \
                            dt_bias, neg_a, Dw, heads, P, N, G, y, state, state_stride, req_start, state_slots, mode,     \
                            chunk_len, max_chunks, scr_s, scr_a);                                                         \
     } while (0)
@@ -338,13 +347,15 @@ static int ssm_launch(int ni, dim3 grid, size_t lds, hipStream_t stream, const f
     return IC_OK;
 }
 
-IC_EXPORT int ic_ssm_scan(const float* xbc, const void* dt_raw, int dt_stride, int dtype, const float* dt_bias,
+IC_EXPORT int ic_ssm_scan(const void* xbc, int x_stride, int x_dtype, int in_act, const void* dt_raw, int dt_stride, int dtype, const float* dt_bias,
                           const float* neg_a, const float* Dw, int heads, int P, int N, int G, float* y, float* state,
                           long long state_stride, const int* req_start, const int* state_slots, int R, int chunk_len,
                           int max_chunks, float* scr_s, float* scr_a, hipStream_t stream) {
     if (R <= 0) return IC_OK;
-    if (heads <= 0 || P <= 0 || P > 256 || N <= 0 || G <= 0 || heads % G || !state) return IC_ERR_ARG;
+    if (heads <= 0 || P <= 0 || P > 256 || N <= 0 || G <= 0 || heads % G || !state || !xbc || !neg_a) return IC_ERR_ARG;
+    if (x_stride < heads * P + 2 * G * N || (x_dtype != IC_F32 && x_dtype != dtype)) return IC_ERR_ARG;
     if (2 * N + P > 1024) return IC_ERR_TOO_LARGE;
+    const int x_f32 = x_dtype == IC_F32;
     const bool chunked = chunk_len > 0 && max_chunks > 1;
     if (chunked && (!scr_s || !scr_a || max_chunks > 65535)) return IC_ERR_ARG;
     const int ngrp = 256 / P, ni = (N + ngrp - 1) / ngrp;
@@ -360,10 +371,10 @@ IC_EXPORT int ic_ssm_scan(const float* xbc, const void* dt_raw, int dt_stride, i
         dim3 grid(heads, R, chunked ? max_chunks : 1);
         int st;
         if (dtype == IC_F32)
-            st = ssm_launch<float>(ni, grid, lds, stream, xbc, dt_raw, dt_stride, dt_bias, neg_a, Dw, heads, P, N, G, y, state,
+            st = ssm_launch<float>(ni, grid, lds, stream, xbc, x_stride, x_f32, in_act, dt_raw, dt_stride, dt_bias, neg_a, Dw, heads, P, N, G, y, state,
                                    state_stride, req_start, state_slots, mode, chunk_len, max_chunks, scr_s, scr_a);
         else if (dtype == IC_BF16)
-            st = ssm_launch<bf16>(ni, grid, lds, stream, xbc, dt_raw, dt_stride, dt_bias, neg_a, Dw, heads, P, N, G, y, state,
+            st = ssm_launch<bf16>(ni, grid, lds, stream, xbc, x_stride, x_f32, in_act, dt_raw, dt_stride, dt_bias, neg_a, Dw, heads, P, N, G, y, state,
                                   state_stride, req_start, state_slots, mode, chunk_len, max_chunks, scr_s, scr_a);
         else
             return IC_ERR_UNSUPPORTED;
@@ -372,39 +383,44 @@ IC_EXPORT int ic_ssm_scan(const float* xbc, const void* dt_raw, int dt_stride, i
     return ic_launch_status();
 }
 
-// ---- gate, then RMS norm in groups ----------------------------------------------------------------------------------
-// v = y * silu(z); every group of `gs` columns is divided by its own root mean square; times w.  One block per
-// (token, group).
+// ---- gate and RMS norm in groups --------------------------------------------------------------------------------------
+// mode 0: v = y * silu(z); every group of `gs` columns is divided by its own root mean square; times w (the gate before
+// the norm).  mode 1: y's groups are divided by their root mean square, times w, times sigmoid(z) (the gate after it).
+// One block per (token, group).
 template <typename T>
 __global__ void __launch_bounds__(256)
 gated_group_norm_kernel(const float* __restrict__ y, const T* __restrict__ z, int z_stride, const float* __restrict__ w,
-                        int inner, int gs, float eps, T* __restrict__ out) {
+                        int inner, int gs, float eps, T* __restrict__ out, int mode) {
     extern __shared__ float v_row[];          // gs floats
     __shared__ float red[8];
     const int t = blockIdx.x, c0 = blockIdx.y * gs;
     float ss = 0.f;
     for (int j = threadIdx.x; j < gs; j += blockDim.x) {
-        const float v = y[(size_t)t * inner + c0 + j] * silu_f(to_f32(z[(size_t)t * z_stride + c0 + j]));
+        float v = y[(size_t)t * inner + c0 + j];
+        if (mode == 0) v *= silu_f(to_f32(z[(size_t)t * z_stride + c0 + j]));
         v_row[j] = v;
         ss += v * v;
     }
     const float r = 1.0f / sqrtf(block_sum(ss, red) / (float)gs + eps);
-    for (int j = threadIdx.x; j < gs; j += blockDim.x)
-        out[(size_t)t * inner + c0 + j] = from_f32<T>(v_row[j] * r * w[c0 + j]);
+    for (int j = threadIdx.x; j < gs; j += blockDim.x) {
+        float v = v_row[j] * r * w[c0 + j];
+        if (mode == 1) v *= sigmoid_f(to_f32(z[(size_t)t * z_stride + c0 + j]));
+        out[(size_t)t * inner + c0 + j] = from_f32<T>(v);
+    }
 }
 
 IC_EXPORT int ic_gated_group_norm(const float* y, const void* z, int z_stride, int dtype, const float* w, int inner,
-                                  int groups, float eps, void* out, int T, hipStream_t stream) {
+                                  int groups, float eps, void* out, int T, int mode, hipStream_t stream) {
     if (T <= 0) return IC_OK;
-    if (inner <= 0 || groups <= 0 || inner % groups || inner / groups > 16128) return IC_ERR_ARG;
+    if (inner <= 0 || groups <= 0 || inner % groups || inner / groups > 16128 || mode < 0 || mode > 1) return IC_ERR_ARG;
     const int gs = inner / groups;
     dim3 grid(T, groups), block(256);
     if (dtype == IC_F32)
         hipLaunchKernelGGL(gated_group_norm_kernel<float>, grid, block, gs * sizeof(float), stream, y, (const float*)z,
-                           z_stride, w, inner, gs, eps, (float*)out);
+                           z_stride, w, inner, gs, eps, (float*)out, mode);
     else if (dtype == IC_BF16)
         hipLaunchKernelGGL(gated_group_norm_kernel<bf16>, grid, block, gs * sizeof(float), stream, y, (const bf16*)z,
-                           z_stride, w, inner, gs, eps, (bf16*)out);
+                           z_stride, w, inner, gs, eps, (bf16*)out, mode);
     else
         return IC_ERR_UNSUPPORTED;
     return ic_launch_status();

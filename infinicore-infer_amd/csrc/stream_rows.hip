@@ -145,7 +145,8 @@ IC_EXPORT int ic_norm_into_stream(const void* y, int y_dtype, const float* bias,
 //   k <- norm(k + bk) -> K plane at slots[t]
 //   v <- v + bv; mix_mode 1: v_keep[t] = v (float32, for later layers of this step);
 //                mix_mode 2: v = (1 - lambda) v + lambda v_keep[t]        -> V plane at slots[t]
-// norm_mode 0: none; 1: every head's dk entries to unit root mean square, times w[dk] (shared by the heads);
+// norm_mode 0: none; 1: every head's dk entries to unit root mean square, times w[dk] (shared by the heads; qw and kw both
+// null: no weight);
 // 2: the whole of q (or k) to unit root mean square, times w[nh * dk] (or w[nkvh * dk]).
 // One wave per (token, head of q, k or v); head sizes up to 512.
 // ---------------------------------------------------------------------------------------------
@@ -180,7 +181,7 @@ qk_norm_store_kernel(const T* __restrict__ rows, int row_stride, const float* __
             for (int j = 0; j < 8; ++j) ss += val[j] * val[j];
             const float r = 1.0f / sqrtf(wave_sum(ss) / (float)dk + eps);
 #pragma unroll
-            for (int j = 0; j < 8; ++j) { const int e = lane + 64 * j; if (e < dk) val[j] = val[j] * r * w[e]; }
+            for (int j = 0; j < 8; ++j) { const int e = lane + 64 * j; if (e < dk) val[j] = val[j] * r * (w ? w[e] : 1.f); }
         } else if (norm_mode == 2) {                      // the sum runs over the whole of q (or k), which every wave reads
             const int p0 = is_q ? 0 : nq, pn = is_q ? nq : nk;
             float ss = 0.f;
@@ -247,7 +248,10 @@ qk_norm_store_vec_kernel(const T* __restrict__ rows, int row_stride, const float
         }
         if (norm_mode == 1) {
             float wv[N];
-            load_floats<N>((is_q ? qw : kw) + j0, wv);
+            if (qw) load_floats<N>((is_q ? qw : kw) + j0, wv);        // no weights: the heads are brought to unit root mean square, no more
+            else
+#pragma unroll
+                for (int i = 0; i < N; ++i) wv[i] = 1.f;
             float ss = 0.f;
 #pragma unroll
             for (int i = 0; i < N; ++i) ss += val[i] * val[i];
@@ -362,7 +366,8 @@ IC_EXPORT int ic_qk_norm_store(const void* rows, int row_stride, int dtype, cons
     if (nh <= 0 || nkvh <= 0 || dk <= 0 || dv <= 0 || page_size <= 0 || norm_mode < 0 || norm_mode > 2 || mix_mode < 0 ||
         mix_mode > 2)
         return IC_ERR_ARG;
-    if (norm_mode != 0 && (qw == nullptr || kw == nullptr)) return IC_ERR_ARG;
+    if ((qw == nullptr) != (kw == nullptr)) return IC_ERR_ARG;
+    if (norm_mode == 2 && qw == nullptr) return IC_ERR_ARG;       // the per-head norm (1) may come without weights
     if (mix_mode != 0 && v_keep == nullptr) return IC_ERR_ARG;
     if (mix_mode == 2 && lambda == nullptr) return IC_ERR_ARG;
     const long long n = (long long)(nh + nkvh) * dk + (long long)nkvh * dv;

@@ -94,6 +94,7 @@ _SIGNATURES = {
     "ic_add_rmsnorm": [_P, _P, _I, _F, _P, _P, _I, _I, _I, _F, _P],
     "ic_residual_add": [_P, _P, _I, _F, _LL, _P],
     "ic_swiglu": [_P, _P, _I, _I, _I, _P],
+    "ic_glu_clamped": [_P, _P, _I, _I, _I, _F, _F, _P],
     "ic_copy_pages": [_P, _I, _LL, _LL, _P, _P, _I, _P],
     "ic_rope_kv_write": [_P, _I, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P],
     "ic_attn_generic": [_P, _I, _P, _I, _I, _P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _F, _I, _P],
@@ -112,19 +113,19 @@ _SIGNATURES = {
     "ic_norm_into_stream": [_P, _I, _P, _P, _P, _P, _I, _I, _I, _F, _P],
     "ic_qk_norm_store": [_P, _I, _I, _P, _P, _P, _I, _F, _I, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P],
     "ic_activation": [_P, _P, _I, _LL, _I, _P],
-    "ic_attn_span_generic": [_P, _I, _P, _I, _P, _I, _I, _P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _I, _I, _P],
+    "ic_attn_span_generic": [_P, _I, _P, _I, _P, _I, _I, _P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _I, _I, _P, _F, _P],
     "ic_attn_span_decode_supported": [_I, _I, _I],
     "ic_attn_span_decode_splits": [_I, _I, _I, _I],
-    "ic_attn_span_decode": [_P, _I, _P, _I, _P, _I, _I, _P, _P, _P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _I, _I, _I, _P],
+    "ic_attn_span_decode": [_P, _I, _P, _I, _P, _I, _I, _P, _P, _P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _I, _I, _P, _F, _I, _P],
     "ic_attn_span_prefill_supported": [_I, _I, _I],
-    "ic_attn_span_prefill": [_P, _I, _P, _I, _P, _I, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _F, _I, _I, _I, _P],
+    "ic_attn_span_prefill": [_P, _I, _P, _I, _P, _I, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _F, _I, _I, _I, _P, _F, _P],
     "ic_pair_rows": [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P],
     "ic_embed_streams": [_P, _P, _P, _P, _I, _P, _I, _I, _I, _P, _P, _P, _P],
     "ic_hc_step": [_P, _I, _I, _I, _P, _I, _P, _P, _P, _P, _F, _P, _I, _P],
     "ic_causal_conv": [_P, _I, _I, _P, _P, _P, _I, _I, _P, _P, _I, _I, _P, _LL, _P, _P, _P, _I, _I, _P],
     "ic_rglru_scan": [_P, _P, _P, _P, _I, _I, _P, _P, _I, _I, _P, _P, _LL, _P, _P, _I, _I, _I, _P, _P, _P],
-    "ic_ssm_scan": [_P, _P, _I, _I, _P, _P, _P, _I, _I, _I, _I, _P, _P, _LL, _P, _P, _I, _I, _I, _P, _P, _P],
-    "ic_gated_group_norm": [_P, _P, _I, _I, _P, _I, _I, _F, _P, _I, _P],
+    "ic_ssm_scan": [_P, _I, _I, _I, _P, _I, _I, _P, _P, _P, _I, _I, _I, _I, _P, _P, _LL, _P, _P, _I, _I, _I, _P, _P, _P],
+    "ic_gated_group_norm": [_P, _P, _I, _I, _P, _I, _I, _F, _P, _I, _I, _P],
     "ic_blocked_product": [_P, _I, _I, _P, _I, _P, _I, _I, _I, _P, _I, _I, _I, _I, _I, _P],
     "ic_latent_prep": [_P, _I, _I, _I, _I, _I, _P, _P, _F, _P, _I, _P, _P, _P, _P, _I, _P],
     "ic_latent_q_rotate": [_P, _I, _I, _I, _I, _I, _I, _P, _I, _P, _P, _I, _I, _P],

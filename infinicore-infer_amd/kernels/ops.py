@@ -125,6 +125,19 @@ def swiglu(gate_up, out):
     return out
 
 
+def glu_clamped(gate_up, out, limit: float, alpha: float):
+    """out[t, j] = g * sigmoid(alpha * g) * (u + 1) with g = min(gate_up[t, j], limit) and
+    u = clamp(gate_up[t, di + j], -limit, limit)."""
+    _dev(gate_up, out)
+    T, di = out.shape
+    _need(tuple(gate_up.shape) == (T, 2 * di) and gate_up.is_contiguous() and out.is_contiguous()
+          and gate_up.dtype == out.dtype, "glu_clamped: layout")
+    _need(limit > 0, "glu_clamped: the limit must be positive")
+    check(get_lib().ic_glu_clamped(gate_up.data_ptr(), out.data_ptr(), dtype_code(out.dtype), T, di, float(limit),
+                                   float(alpha), _stream()), "glu_clamped")
+    return out
+
+
 def copy_pages(planes, src, dst):
     """planes[..., dst[i], :, :, :] = planes[..., src[i], :, :, :] for a cache group's planes
     [slots, planes, pages, kv_heads, page_size, head_dim] (contiguous); src, dst: int32 page ids on the device."""
@@ -701,7 +714,8 @@ def norm_into_stream(y, weight, x, eps: float, bias=None, copy=None):
 
 def qk_norm_store(rows, bias, q_weight, k_weight, norm_mode: int, eps: float, mix_mode: int, mix_lambda, v_keep, q_out,
                   kcache, vcache, slots, n_heads: int, n_kv_heads: int, key_dim: int, value_dim: int, page_size: int):
-    """One pass over the projected rows [q | k | v | ..]: bias, query/key norm (0 none, 1 per head, 2 whole row), value
+    """One pass over the projected rows [q | k | v | ..]: bias, query/key norm (0 none, 1 per head, with weights or with
+    both None to unit root mean square alone, 2 whole row), value
     mixing (0 none, 1 keep the values in ``v_keep``, 2 mix with ``v_keep`` by ``mix_lambda``), q to ``q_out``, k and v
     into the cache planes at ``slots`` (None: no cache write)."""
     _dev(rows, bias, q_weight, k_weight, mix_lambda, v_keep, q_out, kcache, vcache, slots)
@@ -713,7 +727,8 @@ def qk_norm_store(rows, bias, q_weight, k_weight, norm_mode: int, eps: float, mi
                        (k_weight, (key_dim, nk)[norm_mode == 2], "k weight"), (mix_lambda, 1, "lambda")):
         if v is not None:
             _need(v.dtype == torch.float32 and v.is_contiguous() and v.numel() == n, "qk_norm_store: %s must be float32 [%d]" % (what, n))
-    _need(norm_mode == 0 or (q_weight is not None and k_weight is not None), "qk_norm_store: norm weights missing")
+    _need((q_weight is None) == (k_weight is None), "qk_norm_store: the query and key norms have weights both or neither")
+    _need(norm_mode != 2 or q_weight is not None, "qk_norm_store: the whole-row norm needs its weights")
     if mix_mode:
         _need(v_keep is not None and v_keep.dtype == torch.float32 and v_keep.is_contiguous() and v_keep.numel() == T * nv,
               "qk_norm_store: v_keep must be float32 [T, kv_heads * value_dim]")
@@ -761,10 +776,23 @@ def _span_common(q, out, gate, kcache, vcache, block_tables, n_heads, n_kv_heads
     _need(n_heads % n_kv_heads == 0, "span attention: heads not a multiple of kv heads")
 
 
+def _sink_args(sink, n_heads: int):
+    """``sink``: False (none), True (the term exp(0)) or a float32 tensor [heads] of learned sinks (the term exp(sink_h))."""
+    if isinstance(sink, torch.Tensor):
+        _dev(sink)
+        _need(sink.dtype == torch.float32 and sink.is_contiguous() and sink.numel() == n_heads,
+              "span attention: learned sinks must be float32 [%d]" % n_heads)
+        return 1, sink.data_ptr()
+    return int(bool(sink)), None
+
+
 def attention_span_generic(q, out, gate, kcache, vcache, block_tables, token_req, positions, n_heads, n_kv_heads, key_dim,
-                           value_dim, page_size, scale: float, window: int = 0, keep_first: int = 0, sink: bool = False):
+                           value_dim, page_size, scale: float, window: int = 0, keep_first: int = 0, sink=False,
+                           softcap: float = 0.0):
     """out[t, h] = sum_j p_j V_j over the keys j <= positions[t] with positions[t] - j < window or j < keep_first
-    (window 0: all), p = softmax of scale * q . K_j with ``sink`` added to the denominator; times sigmoid(gate)."""
+    (window 0: all), p = softmax of s_j = scale * q . K_j (``softcap`` c > 0: s_j <- c tanh(s_j / c)) with the sink's
+    term added to the denominator (``sink``: see ``_sink_args``); times sigmoid(gate)."""
+    sink_flag, sink_ptr = _sink_args(sink, n_heads)
     _span_common(q, out, gate, kcache, vcache, block_tables, n_heads, n_kv_heads, key_dim, value_dim, page_size)
     _i32(token_req, "token_req")
     _i32(positions, "positions")
@@ -775,7 +803,8 @@ def attention_span_generic(q, out, gate, kcache, vcache, block_tables, token_req
         q.data_ptr(), q.stride(0), out.data_ptr(), out.stride(0), gate.data_ptr() if gate is not None else None,
         gate.stride(0) if gate is not None else 0, dtype_code(q.dtype), kcache.data_ptr(), vcache.data_ptr(),
         block_tables.data_ptr(), block_tables.stride(0), token_req.data_ptr(), positions.data_ptr(), T, n_heads, n_kv_heads,
-        key_dim, value_dim, page_size, float(scale), int(window or 0), int(keep_first or 0), int(bool(sink)), _stream()),
+        key_dim, value_dim, page_size, float(scale), int(window or 0), int(keep_first or 0), sink_flag, sink_ptr,
+        float(softcap or 0.0), _stream()),
         "attention_span_generic")
 
 
@@ -790,7 +819,7 @@ def attention_span_decode_splits(n_rows: int, n_kv_heads: int, max_keys: int, co
 
 def attention_span_decode(q, out, gate, kcache, vcache, block_tables, tok_list, n_tok, token_req, positions, part_acc,
                           part_ml, n_heads, n_kv_heads, key_dim, value_dim, page_size, scale: float, window: int = 0,
-                          keep_first: int = 0, sink: bool = False, n_split: int = 1):
+                          keep_first: int = 0, sink=False, softcap: float = 0.0, n_split: int = 1):
     """The rows ``tok_list`` (None: rows 0..n_tok-1) of q, each a request's single new token, split ``n_split`` ways
     over their visible keys.  part_acc / part_ml: float32 scratch of n_tok * heads * n_split * (value_dim / 2) elements."""
     _span_common(q, out, gate, kcache, vcache, block_tables, n_heads, n_kv_heads, key_dim, value_dim, page_size)
@@ -802,6 +831,7 @@ def attention_span_decode(q, out, gate, kcache, vcache, block_tables, tok_list, 
     else:
         _need(n_tok <= q.shape[0], "span decode: more tokens than rows")
     _need(1 <= n_split <= 32, "span decode: 1..32 splits")
+    sink_flag, sink_ptr = _sink_args(sink, n_heads)
     if n_split > 1:
         _dev(part_acc, part_ml)
         _need(part_acc.dtype == torch.float32 and part_ml.dtype == torch.float32
@@ -813,7 +843,8 @@ def attention_span_decode(q, out, gate, kcache, vcache, block_tables, tok_list, 
         block_tables.data_ptr(), block_tables.stride(0), tok_list.data_ptr() if tok_list is not None else None,
         token_req.data_ptr(), positions.data_ptr(), part_acc.data_ptr() if n_split > 1 else None,
         part_ml.data_ptr() if n_split > 1 else None, n_tok, n_heads, n_kv_heads, key_dim, value_dim, page_size,
-        float(scale), int(window or 0), int(keep_first or 0), int(bool(sink)), int(n_split), _stream()),
+        float(scale), int(window or 0), int(keep_first or 0), sink_flag, sink_ptr, float(softcap or 0.0), int(n_split),
+        _stream()),
         "attention_span_decode")
 
 
@@ -823,8 +854,10 @@ def attention_span_prefill_supported(dtype, key_dim: int, value_dim: int) -> boo
 
 
 def attention_span_prefill(q, out, gate, kcache, vcache, block_tables, tiles, n_tiles, n_heads, n_kv_heads, key_dim,
-                           value_dim, page_size, scale: float, window: int = 0, keep_first: int = 0, sink: bool = False):
+                           value_dim, page_size, scale: float, window: int = 0, keep_first: int = 0, sink=False,
+                           softcap: float = 0.0):
     """Prompt portions listed as tiles int32 [n_tiles, 4] (request row, first token row, rows, first position)."""
+    sink_flag, sink_ptr = _sink_args(sink, n_heads)
     _span_common(q, out, gate, kcache, vcache, block_tables, n_heads, n_kv_heads, key_dim, value_dim, page_size)
     _dev(tiles)
     _need(tiles.dtype == torch.int32 and tiles.is_contiguous() and tiles.numel() >= 4 * n_tiles, "span prefill: tiles layout")
@@ -833,7 +866,8 @@ def attention_span_prefill(q, out, gate, kcache, vcache, block_tables, tiles, n_
         q.data_ptr(), q.stride(0), out.data_ptr(), out.stride(0), gate.data_ptr() if gate is not None else None,
         gate.stride(0) if gate is not None else 0, dtype_code(q.dtype), kcache.data_ptr(), vcache.data_ptr(),
         block_tables.data_ptr(), block_tables.stride(0), tiles.data_ptr(), n_tiles, n_heads, n_kv_heads, key_dim, value_dim,
-        page_size, float(scale), int(window or 0), int(keep_first or 0), int(bool(sink)), _stream()),
+        page_size, float(scale), int(window or 0), int(keep_first or 0), sink_flag, sink_ptr, float(softcap or 0.0),
+        _stream()),
         "attention_span_prefill")
 
 
@@ -968,36 +1002,49 @@ def rglru_scan(gates, gate_bias, u, yb, y_bias, decay, block_width: int, out, st
 
 
 def ssm_scan(xbc, dt_raw, dt_bias, neg_a, d_skip, heads: int, head_dim: int, state_dim: int, groups: int, y, state,
-             state_offset: int, req_start, state_slots, n_requests: int, chunks=None):
-    """The state-space recurrence over every request's rows (see csrc/recurrent.hip): y float32 [T, heads * head_dim]."""
+             state_offset: int, req_start, state_slots, n_requests: int, chunks=None, in_act=None):
+    """The state-space recurrence over every request's rows (see csrc/recurrent.hip): y float32 [T, heads * head_dim].
+    ``xbc`` [T, >= inner + 2 groups state_dim] holds x, B, C of every token, float32 or y's compute dtype (rows may be
+    strided: a projection's own columns); ``in_act`` "silu": applied as they are read.  ``dt_raw`` None: no step sizes,
+    ``neg_a`` is then the fixed decay per head and every step is one (linear attention with keys B, values x, queries
+    C); ``dt_bias`` and ``d_skip`` may be None."""
     _dev(xbc, dt_raw, dt_bias, neg_a, d_skip, y, state, req_start, state_slots)
     T = xbc.shape[0]
     inner = heads * head_dim
-    _need(xbc.dtype == torch.float32 and xbc.is_contiguous() and xbc.shape[1] == inner + 2 * groups * state_dim, "ssm_scan: xbc")
+    _need(xbc.dim() == 2 and xbc.stride(1) == 1 and xbc.shape[1] >= inner + 2 * groups * state_dim
+          and xbc.stride(0) >= inner + 2 * groups * state_dim, "ssm_scan: xbc")
     _need(y.dtype == torch.float32 and y.is_contiguous() and tuple(y.shape) == (T, inner), "ssm_scan: y")
-    _need(tuple(dt_raw.shape) == (T, heads) and dt_raw.stride(1) == 1, "ssm_scan: dt")
+    _need(in_act in (None, "silu"), "ssm_scan: in_act is None or 'silu'")
+    if dt_raw is not None:
+        _need(tuple(dt_raw.shape) == (T, heads) and dt_raw.stride(1) == 1, "ssm_scan: dt")
+        _need(xbc.dtype in (torch.float32, dt_raw.dtype), "ssm_scan: xbc is float32 or of the step sizes' dtype")
     for v in (dt_bias, neg_a, d_skip):
-        _need(v.dtype == torch.float32 and v.numel() == heads and v.is_contiguous(), "ssm_scan: per-head vectors")
+        _need(v is None or (v.dtype == torch.float32 and v.numel() == heads and v.is_contiguous()), "ssm_scan: per-head vectors")
+    _need(neg_a is not None, "ssm_scan: the decays are missing")
     _i32(req_start, "req_start")
     _i32(state_slots, "state_slots")
     sp, stride = _state_part(state, state_offset)
     _need(state_offset + inner * state_dim <= stride, "ssm_scan: state too small")
-    check(get_lib().ic_ssm_scan(xbc.data_ptr(), dt_raw.data_ptr(), dt_raw.stride(0), dtype_code(dt_raw.dtype), dt_bias.data_ptr(),
-                                neg_a.data_ptr(), d_skip.data_ptr(), heads, head_dim, state_dim, groups, y.data_ptr(), sp, stride,
+    dt_code = dtype_code(dt_raw.dtype) if dt_raw is not None else dtype_code(xbc.dtype)
+    check(get_lib().ic_ssm_scan(xbc.data_ptr(), xbc.stride(0), dtype_code(xbc.dtype), 1 if in_act else 0, _ptr(dt_raw),
+                                dt_raw.stride(0) if dt_raw is not None else 0, dt_code, _ptr(dt_bias),
+                                neg_a.data_ptr(), _ptr(d_skip), heads, head_dim, state_dim, groups, y.data_ptr(), sp, stride,
                                 req_start.data_ptr(), state_slots.data_ptr(), n_requests,
                                 *_chunk_scratch(chunks, inner * state_dim, heads, n_requests, "ssm_scan"), _stream()), "ssm_scan")
     return y
 
 
-def gated_group_norm(y, z, weight, groups: int, eps: float, out):
-    """out = rms_in_groups(y * silu(z)) * weight; y float32 [T, n], z and out the compute dtype."""
+def gated_group_norm(y, z, weight, groups: int, eps: float, out, gate_after: bool = False):
+    """out = rms_in_groups(y * silu(z)) * weight, or with ``gate_after`` rms_in_groups(y) * weight * sigmoid(z);
+    y float32 [T, n], z (rows may be strided) and out the compute dtype."""
     _dev(y, z, weight, out)
     T, n = y.shape
     _need(y.dtype == torch.float32 and y.is_contiguous() and tuple(z.shape) == (T, n) and z.stride(1) == 1
           and out.dtype == z.dtype and tuple(out.shape) == (T, n) and out.is_contiguous(), "gated_group_norm: layout")
     _need(weight.dtype == torch.float32 and weight.numel() == n and weight.is_contiguous(), "gated_group_norm: weight")
     check(get_lib().ic_gated_group_norm(y.data_ptr(), z.data_ptr(), z.stride(0), dtype_code(z.dtype), weight.data_ptr(), n,
-                                        int(groups), float(eps), out.data_ptr(), T, _stream()), "gated_group_norm")
+                                        int(groups), float(eps), out.data_ptr(), T, 1 if gate_after else 0, _stream()),
+          "gated_group_norm")
     return out
 
 

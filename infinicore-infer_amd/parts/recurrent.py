@@ -7,8 +7,11 @@
 ``mamba2``: a state-space recurrence with a matrix state [N, P] per head.  W_in h = [z | x | B | C | dt]; x, B, C pass
     a causal convolution per channel and silu; dt = softplus(dt + dt_bias);
     S_t = exp(-exp(A_log) dt) S_(t-1) + dt B x^T,   y = S^T C + D x;   out = W_o (rms_in_groups(y silu(z)) * w).
-Both keep, beside the recurrent state, the convolution's last taps - 1 inputs; one float32 vector per request holds the two.
-The state starts at zero.  Products run in the compute dtype; gates, decays, step sizes and the state are float32.
+``decay_linear_attention``: linear attention with a fixed decay per head and a matrix state [dim, vdim] per head.
+    q = silu(W_q h), k = silu(W_k h), v = silu(W_v h);   S_t = decay_h S_(t-1) + k_t v_t^T,   o_t = S_t^T q_t;
+    out = W_o (rms(o) * w * sigmoid(W_g h))    (the norm over all heads together, the gate after it).
+The first two keep, beside the recurrent state, the convolution's last taps - 1 inputs; one float32 vector per request holds
+the two.  The state starts at zero.  Products run in the compute dtype; gates, decays, step sizes and the state are float32.
 """
 import torch
 
@@ -165,6 +168,70 @@ class StateSpaceMixer(Mixer):
                      cache.state, 0, *lists, chunks=chunk_plan(ctx, inner * self.N, self.heads, "ssm"))
         g = ctx.ws.buffer("ssm_gated", (T, inner), rt.dtype)
         ops.gated_group_norm(y, proj[:, :inner], self.norm_w, self.norm_groups, self.eps, g)
+        out = ctx.ws.buffer("mixer_out", (T, self.hidden_size), rt.dtype)
+        linear(g, self.w_o, out, rt.gemm_impl, ws=ctx.ws)
+        return out
+
+
+@register_part("mixer", "decay_linear_attention")
+class DecayLinearAttention(Mixer):
+    """Linear attention whose state decays by a fixed factor per head.  The recurrence is the state-space one with keys
+    for B, values for x, queries for C, one group per head, steps of one and no skip term, so it runs in the same scan
+    kernel (single pass for few tokens, chunks side by side for prompt portions), which reads q, k, v straight from the
+    projection's rows and applies their silu on the way in.  The four matrices are one projection, laid out [v | k | q | g]."""
+    graph_safe = True
+
+    def __init__(self, name, runtime, hidden_size: int, heads: int, key_dim: int, value_dim: int, decay, norm_eps: float):
+        super().__init__(name, runtime)
+        decay = [float(a) for a in decay]
+        if heads <= 0 or len(decay) != heads:
+            raise ValueError("linear attention: %d heads but %d decays" % (heads, len(decay)))
+        if any(not 0.0 <= a <= 1.0 for a in decay):
+            raise ValueError("linear attention: a decay lies outside [0, 1]")
+        if not 0 < value_dim <= 256:
+            raise ValueError("linear attention: a head's value size must lie in 1..256 (got %d)" % value_dim)
+        if key_dim <= 0 or 2 * key_dim + value_dim > 1024 or -(-key_dim // (256 // value_dim)) > 128:
+            raise ValueError("linear attention: a head's state of %d x %d is beyond what the kernel keeps in registers" % (key_dim, value_dim))
+        self.hidden_size, self.heads, self.dk, self.dv = int(hidden_size), int(heads), int(key_dim), int(value_dim)
+        self.eps = float(norm_eps)
+        self.nq, self.nv = self.heads * self.dk, self.heads * self.dv
+        self.proj = 2 * self.nq + 2 * self.nv
+        self.state_size = self.heads * self.dk * self.dv
+        self.decay = torch.tensor(decay, dtype=torch.float64).to(torch.float32).to(runtime.device)
+
+    def cache_need(self):
+        return CacheNeed("state", state_shape=(self.state_size,), state_dtype=torch.float32)
+
+    def weight_specs(self):
+        n, d = self.name, self.hidden_size
+        pack = n + "vkqg.packed"
+        return {
+            n + "v": WeightSpec((self.nv, d), pack=(pack, 0)), n + "k": WeightSpec((self.nq, d), pack=(pack, 1)),
+            n + "q": WeightSpec((self.nq, d), pack=(pack, 2)), n + "g": WeightSpec((self.nv, d), pack=(pack, 3)),
+            n + "norm": WeightSpec((self.nv,), "vector"),
+            n + "o": WeightSpec((d, self.nv)),
+        }
+
+    def load_weights(self, tensors):
+        n = self.name
+        packed = tensors.get(n + "vkqg.packed")
+        if packed is None:
+            mats = [tensors[n + s] for s in ("v", "k", "q", "g")]
+            if len({m.dtype for m in mats}) > 1:
+                mats = [m.to(torch.float32) for m in mats]
+            packed = torch.cat(mats, dim=0).contiguous()
+        self.w_rows, self.w_o, self.norm_w = packed, tensors[n + "o"], tensors[n + "norm"]
+
+    def forward(self, h, ctx, cache):
+        rt, T = self.runtime, h.shape[0]
+        rows = ctx.ws.buffer("linattn_rows", (T, self.proj), rt.dtype)
+        linear(h, self.w_rows, rows, rt.gemm_impl, ws=ctx.ws)
+        o = ctx.ws.buffer("linattn_o", (T, self.nv), torch.float32)
+        ops.ssm_scan(rows, None, None, self.decay, None, self.heads, self.dv, self.dk, self.heads, o, cache.state, 0,
+                     ctx.req_rows, ctx.state_slots, ctx.R, chunks=chunk_plan(ctx, self.state_size, self.heads, "linattn"),
+                     in_act="silu")
+        g = ctx.ws.buffer("linattn_gated", (T, self.nv), rt.dtype)
+        ops.gated_group_norm(o, rows[:, self.nv + 2 * self.nq:], self.norm_w, 1, self.eps, g, gate_after=True)
         out = ctx.ws.buffer("mixer_out", (T, self.hidden_size), rt.dtype)
         linear(g, self.w_o, out, rt.gemm_impl, ws=ctx.ws)
         return out

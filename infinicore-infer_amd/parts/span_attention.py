@@ -5,8 +5,11 @@ scores.  Options, each a parameter:
 
   * biases on the q, k, v projections and on the output projection,
   * a norm on queries and keys to unit root mean square, per head (one weight of the key size, shared by the
-    heads) or over the whole projection before it is cut into heads (a weight of the projection's size),
-  * a sink: one more term exp(0) in the softmax's denominator that has no value, p_j = e^{s_j} / (1 + sum e^{s_j}),
+    heads, or no weight at all) or over the whole projection before it is cut into heads (a weight of the
+    projection's size),
+  * a cap on the scaled score, s <- c tanh(s / c),
+  * a sink: one more term in the softmax's denominator that has no value, p_j = e^{s_j} / (e^{z} + sum e^{s_j}),
+    with z = 0 or z a learned number per head (the tensor ``sink``), neither scaled nor capped,
   * value mixing: the first mixing layer of the model keeps its values of the step's tokens, every later one
     replaces its own by (1 - lambda) v + lambda v_first before they are cached (lambda a learned scalar),
   * an output gate: the concatenated heads are multiplied by sigmoid(W_g h) before the output projection.
@@ -34,8 +37,11 @@ class SpanAttention(Mixer):
     def __init__(self, name, runtime, hidden_size: int, num_heads: int, num_kv_heads: int, key_dim: int,
                  value_dim: int, softmax_scale: float, window=None, keep_first: int = 0, sink: bool = False,
                  qk_norm=None, qk_norm_eps: float = 1e-6, qkv_bias: bool = False, out_bias: bool = False,
-                 gate: bool = False, value_mix=None, value_mix_width=None, value_mix_optional: bool = False):
-        """``qk_norm``: None, "head" or "row".  ``value_mix``: None, "keep" (this layer's values are the ones later
+                 gate: bool = False, value_mix=None, value_mix_width=None, value_mix_optional: bool = False,
+                 softcap=None, qk_norm_weight: bool = True):
+        """``sink``: False, True (the constant term exp(0)) or "learned" (one number per head, the tensor ``sink``).
+        ``softcap``: None or the cap c > 0.  ``qk_norm_weight`` False: the per-head norm has no weight tensors.
+        ``qk_norm``: None, "head" or "row".  ``value_mix``: None, "keep" (this layer's values are the ones later
         layers mix in) or "mix"; all mixing layers of a model have the same kv heads and value size.
         ``value_mix_optional``: the files may hold the mixing scalar although this layer does not mix."""
         super().__init__(name, runtime)
@@ -52,7 +58,17 @@ class SpanAttention(Mixer):
         self.keep_first = int(keep_first or 0) if self.window else 0
         if self.keep_first < 0:
             raise ValueError("span attention: keep_first must not be negative")
+        if sink not in (False, True, None, "learned"):
+            raise ValueError("span attention: sink is False, True or 'learned' (got %r)" % (sink,))
         self.sink = bool(sink)
+        self.sink_learned = sink == "learned"
+        self.softcap = float(softcap) if softcap else 0.0
+        if self.softcap < 0:
+            raise ValueError("span attention: the score cap must be positive")
+        self.norm_weight = bool(qk_norm_weight)
+        if not self.norm_weight and qk_norm == "row":
+            raise ValueError("span attention: the norm over the whole projection comes with a weight")
+        self.sinks = None
         self.norm_mode = _NORM_MODES[qk_norm]
         self.qk_norm_eps = float(qk_norm_eps)
         self.qkv_bias, self.out_bias, self.gate = bool(qkv_bias), bool(out_bias), bool(gate)
@@ -87,7 +103,9 @@ class SpanAttention(Mixer):
             specs[n + "v.b"] = WeightSpec((self.nv,), "vector", pack=(bpack, 2), mean=0.0)
         if self.out_bias:
             specs[n + "o.b"] = WeightSpec((d,), "vector", mean=0.0)
-        if self.norm_mode:
+        if self.sink_learned:
+            specs[n + "sink"] = WeightSpec((self.nh,), "vector", mean=0.0)
+        if self.norm_mode and self.norm_weight:
             per_head = self.norm_mode == 1
             specs[n + "q.norm"] = WeightSpec((self.dk if per_head else self.nq,), "vector")
             specs[n + "k.norm"] = WeightSpec((self.dk if per_head else self.nk,), "vector")
@@ -113,8 +131,10 @@ class SpanAttention(Mixer):
                 b = torch.cat([tensors[n + s + ".b"].to(torch.float32).reshape(-1) for s in ("q", "k", "v")]).contiguous()
             self.b_rows = b
         self.b_o = tensors[n + "o.b"] if self.out_bias else None
-        if self.norm_mode:
+        if self.norm_mode and self.norm_weight:
             self.q_norm, self.k_norm = tensors[n + "q.norm"], tensors[n + "k.norm"]
+        if self.sink_learned:
+            self.sinks = tensors[n + "sink"].to(torch.float32).contiguous()
         if self.mix_mode == 2:
             self.mix_lambda = tensors[n + "vmix"].reshape(1)
 
@@ -145,7 +165,8 @@ class SpanAttention(Mixer):
         """Single-token rows go to the split-key kernel, prompt portions to the matrix-core kernel, where the sizes
         have one (and the runtime does not ask for the general kernel alone); everything else to the general kernel."""
         rt = self.runtime
-        args = (self.nh, self.nkvh, self.dk, self.dv, ctx.page_size, self.scale, self.window, self.keep_first, self.sink)
+        args = (self.nh, self.nkvh, self.dk, self.dv, ctx.page_size, self.scale, self.window, self.keep_first,
+                self.sinks if self.sink_learned else self.sink, self.softcap)
         n_dec, n_tiles = ctx.n_decode_rows, ctx.n_prefill_tiles
         tiled = rt.attention_impl == "auto" and n_dec + n_tiles > 0
         use_dec = tiled and n_dec > 0 and ops.attention_span_decode_supported(rt.dtype, self.dk, self.dv)

@@ -1,4 +1,5 @@
-"""Dense SwiGLU feed-forward: down( up(h) * silu(gate(h)) ).
+"""Dense gated feed-forward: down( up(h) * silu(gate(h)) ), or with ``variant="clamped"`` the unit with bounded
+branches, g = min(gate(h), limit), u = clamp(up(h), -limit, limit), down( g sigmoid(alpha g) (u + 1) ).
 
 The reference fuses gate and up into one projection with rows [gate; up]
 (scripts/jiuge.py:311-323), applies swiglu(out=gate, up, gate)
@@ -20,9 +21,16 @@ class SwiGLU(FeedForward):
     fuses_tail = True
 
     def __init__(self, name, runtime, hidden_size: int, intermediate_size: int, gate_name: str = "gate_proj.weight",
-                 up_name: str = "up_proj.weight", down_name: str = "down_proj.weight"):
-        """``gate_name`` / ``up_name`` / ``down_name``: the matrices' names after the part's prefix."""
+                 up_name: str = "up_proj.weight", down_name: str = "down_proj.weight", variant: str = "silu",
+                 limit=None, alpha: float = 1.0):
+        """``gate_name`` / ``up_name`` / ``down_name``: the matrices' names after the part's prefix.  ``variant``: "silu"
+        or "clamped" (with its ``limit`` > 0 and the sigmoid's slope ``alpha``)."""
         super().__init__(name, runtime)
+        if variant not in ("silu", "clamped"):
+            raise ValueError("gated feed-forward: variant %r (have silu, clamped)" % (variant,))
+        if variant == "clamped" and not (limit is not None and float(limit) > 0):
+            raise ValueError("gated feed-forward: the clamped unit needs a positive limit")
+        self.variant, self.limit, self.alpha = variant, (float(limit) if limit is not None else None), float(alpha)
         self.hidden_size = hidden_size
         self.intermediate_size = intermediate_size
         self.gate_name, self.up_name, self.down_name = name + gate_name, name + up_name, name + down_name
@@ -52,7 +60,7 @@ class SwiGLU(FeedForward):
     def native_desc(self):
         from ..kernels.lib import IcSwiGLU
         ws = (self.w_gate_up, self.w_down)
-        if not (self._forward_is(SwiGLU)
+        if not (self._forward_is(SwiGLU) and self.variant == "silu"
                 and all(w is not None and w.is_cuda and w.dtype == self.runtime.dtype and w.is_contiguous() for w in ws)):
             return None
         return IcSwiGLU(self.intermediate_size, self.w_gate_up.data_ptr(), self.w_down.data_ptr())
@@ -65,7 +73,7 @@ class SwiGLU(FeedForward):
         act = ctx.ws.buffer("ffn_act", (T, self.intermediate_size), rt.dtype)
         owed = isinstance(h, DeferredRows)
         rows = h.values if owed else h
-        few = (rt.gemm_impl == "auto" and rows.dtype == self.w_gate_up.dtype == act.dtype
+        few = (self.variant == "silu" and rt.gemm_impl == "auto" and rows.dtype == self.w_gate_up.dtype == act.dtype
                and ops.rule_gate_up_fused(rows.dtype, T, rows, self.w_gate_up, owed))
         if few:
             # few rows: the activation is the epilogue of the gate/up projection
@@ -76,7 +84,10 @@ class SwiGLU(FeedForward):
         else:
             gate_up = ctx.ws.buffer("gate_up", (T, 2 * self.intermediate_size), rt.dtype)
             linear(h, self.w_gate_up, gate_up, rt.gemm_impl, ws=ctx.ws)
-            ops.swiglu(gate_up, act)
+            if self.variant == "clamped":
+                ops.glu_clamped(gate_up, act, self.limit, self.alpha)
+            else:
+                ops.swiglu(gate_up, act)
         fused = linear_tail(act, self.w_down, tail, ctx.ws, "ffn_tail", rt.gemm_impl)
         if fused is not None:
             return fused
