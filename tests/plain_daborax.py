@@ -96,26 +96,44 @@ def lightning_mixer(h, W, p, heads, dim, vdim, decay, eps):
 
 
 # ---- softmax attention over a window, with a capped score and a learned sink ---------------------------------
+def seen(n_queries, n_keys, window, first=0):
+    """[queries, keys] True where query at position first + i sees key j: 0 <= (first + i) - j < window (no window: all earlier keys)."""
+    i = torch.arange(first, first + n_queries)[:, None]
+    j = torch.arange(n_keys)[None, :]
+    ok = j <= i
+    return ok if window is None else ok & (i - j < window)
+
+
+def sink_softmax(scores, mask, sink, softcap=None):
+    """Weights of the seen keys: the score is capped (cap * tanh(score / cap)), then exp(score) / (exp(sink) + sum exp(score));
+    the sink has no key and is neither capped nor scaled.  ``sink`` None: a plain softmax."""
+    if softcap:
+        scores = softcap * torch.tanh(scores / softcap)
+    scores = scores.masked_fill(~mask, float("-inf"))
+    m = scores.max(-1, keepdim=True).values
+    if sink is not None:
+        m = torch.maximum(m, torch.as_tensor(sink, dtype=scores.dtype))
+    e = torch.exp(scores - m)
+    den = e.sum(-1, keepdim=True)
+    if sink is not None:
+        den = den + torch.exp(torch.as_tensor(sink, dtype=scores.dtype) - m)
+    return e / den
+
+
 def window_attention(h, W, p, heads, kv_heads, dim, vdim, scale, softcap, window, eps):
     T = h.shape[0]
     q = (h @ W[p + "q"].T + W[p + "q.b"]).reshape(T, heads, dim)
     k = (h @ W[p + "k"].T + W[p + "k.b"]).reshape(T, kv_heads, dim)
     v = (h @ W[p + "v"].T + W[p + "v.b"]).reshape(T, kv_heads, vdim)
     q, k = unit_rms(q, eps), unit_rms(k, eps)
-    out = torch.zeros(T, heads, vdim, dtype=h.dtype)
+    mask = seen(T, T, window)
     per = heads // kv_heads
+    out = []
     for hd in range(heads):
         g = hd // per
-        for i in range(T):
-            lo = 0 if window is None else max(0, i - window + 1)
-            s = (k[lo:i + 1, g] @ q[i, hd]) * scale
-            if softcap:
-                s = softcap * torch.tanh(s / softcap)
-            sink = W[p + "sink"][hd]
-            m = torch.maximum(s.max(), sink)
-            e = torch.exp(s - m)
-            out[i, hd] = (e[:, None] * v[lo:i + 1, g]).sum(0) / (e.sum() + torch.exp(sink - m))
-    return out.reshape(T, heads * vdim) @ W[p + "o"].T + W[p + "o.b"]
+        w = sink_softmax((q[:, hd] @ k[:, g].T) * scale, mask, W[p + "sink"][hd], softcap)
+        out.append(w @ v[:, g])
+    return torch.cat(out, -1) @ W[p + "o"].T + W[p + "o.b"]
 
 
 # ---- feed-forward -----------------------------------------------------------------------------------------
@@ -141,8 +159,8 @@ def run_mixer(h, W, p, kind, m, eps):
 def forward(cfg, W, tokens, dtype=torch.float64, layers_out=None):
     """Logits [T, vocab] of one whole sequence.  ``layers_out``: a list that receives the residual stream after every layer."""
     W = {k: (v.to(dtype) if v.is_floating_point() else v) for k, v in W.items()}
-    eps, mult = cfg["norm"]["eps"], cfg["residual_mult"]
-    x = embed(tokens, W["embed"], cfg["embedding"]["scale"])
+    eps, mult = cfg["norm"]["eps"], cfg.get("residual_mult", 1.0)
+    x = embed(tokens, W["embed"], (cfg.get("embedding") or {}).get("scale", 1.0))
     for i, l in enumerate(cfg["layers"]):
         src = l.get("weights_of", i)
         src = i if src is None else src
@@ -155,3 +173,43 @@ def forward(cfg, W, tokens, dtype=torch.float64, layers_out=None):
         if layers_out is not None:
             layers_out.append(x.clone())
     return (unit_rms(x, eps) * W["final.norm"]) @ W["head"].T
+
+
+# ---- random weights for the tests ---------------------------------------------------------------------------------
+def random_weights(cfg, seed, std=1.0):
+    """Every tensor of a configuration, float32: matrices with entries of size std / sqrt(inputs), norm weights and layer
+    scales around one, biases, sinks and the recurrences' vectors of order one."""
+    g = torch.Generator().manual_seed(seed)
+    d = cfg["width"]
+    lin = lambda o, i: torch.randn(o, i, generator=g) * (std / math.sqrt(i))
+    around_one = lambda n: 1.0 + 0.2 * torch.randn(n, generator=g)
+    W = {"embed": 0.5 * torch.randn(cfg["vocab"], d, generator=g), "head": lin(cfg["vocab"], d), "final.norm": around_one(d)}
+    for i, l in enumerate(cfg["layers"]):
+        if l.get("weights_of") is not None:
+            continue
+        p, m = "l%d." % i, l["mixer"]
+        W[p + "norm1"], W[p + "ls1"] = around_one(d), 0.5 + torch.rand(d, generator=g)
+        if l["type"] == "attention":
+            H, G = m["heads"], m.get("kv_heads") or m["heads"]
+            dk, dv = m["dim"], m.get("vdim") or m["dim"]
+            W[p + "mix.q"], W[p + "mix.k"], W[p + "mix.v"] = lin(H * dk, d), lin(G * dk, d), lin(G * dv, d)
+            W[p + "mix.q.b"], W[p + "mix.k.b"], W[p + "mix.v.b"] = (0.3 * torch.randn(n, generator=g) for n in (H * dk, G * dk, G * dv))
+            W[p + "mix.sink"] = torch.randn(H, generator=g)
+            W[p + "mix.o"], W[p + "mix.o.b"] = lin(d, H * dv), 0.3 * torch.randn(d, generator=g)
+        elif l["type"] == "lightning":
+            H, dk, dv = m["heads"], m["dim"], m.get("vdim") or m["dim"]
+            W[p + "mix.q"], W[p + "mix.k"], W[p + "mix.v"], W[p + "mix.g"] = lin(H * dk, d), lin(H * dk, d), lin(H * dv, d), lin(H * dv, d)
+            W[p + "mix.norm"], W[p + "mix.o"] = around_one(H * dv), lin(d, H * dv)
+        else:
+            H, P_, N, G = m["heads"], m["vdim"], m["state"], m["groups"]
+            inner, ch = H * P_, H * P_ + 2 * G * N
+            W[p + "mix.in"] = lin(2 * inner + 2 * G * N + H, d)
+            W[p + "mix.conv"] = torch.randn(ch, m["conv"], generator=g) / math.sqrt(m["conv"])
+            W[p + "mix.conv.b"] = 0.2 * torch.randn(ch, generator=g)
+            W[p + "mix.dt_bias"], W[p + "mix.A_log"] = torch.randn(H, generator=g) - 1.0, 0.5 * torch.randn(H, generator=g)
+            W[p + "mix.D"], W[p + "mix.norm"], W[p + "mix.o"] = torch.randn(H, generator=g), around_one(inner), lin(d, inner)
+        if l.get("mlp"):
+            ff = l["mlp"]["ff"]
+            W[p + "norm2"], W[p + "ls2"] = around_one(d), 0.5 + torch.rand(d, generator=g)
+            W[p + "mlp.gate"], W[p + "mlp.up"], W[p + "mlp.down"] = 2.0 * lin(ff, d), 2.0 * lin(ff, d), lin(d, ff)
+    return {k: v.to(torch.bfloat16).to(torch.float32) for k, v in W.items()}      # what a bfloat16 file holds
