@@ -12,7 +12,7 @@ seeded uniform-random token ids.  One JSON line is printed.
   --workload mixed   the 1B shape's workload: 64 requests, prompts of 128..2,048 tokens, portions of 512
   --workload long    the 8B shape's workload: 4 prompts of 16,384 tokens, then decoding
   --direct           decode by calling the step function directly, without the scheduler
-  --workload designs the Fopezen and Mezinex decoders beside the MiniCPM decoder at equal layer sizes (a few layers of three real
+  --workload designs the Fopezen, Mezinex and Daborax decoders beside the MiniCPM decoder at equal layer sizes (a few layers of three real
                      models' sizes): prefill and decode throughput of both, with the fraction of the memory or
                      matrix-core peak each reaches (--only fopezen|minicpm|mezinex: one of them, for a profiler)
 """
@@ -213,7 +213,22 @@ def _design_configs(z, layers):
                embedding=dict(bigram=dict(buckets=65521, mul_prev=127, mul_cur=17)),
                layers=[dict(type=mez_kinds[i % 4][0], mixer=mez_kinds[i % 4][1], mlp=dict(kind="dense", ff=z["ff"]))
                        for i in range(layers)])
-    return {"minicpm": mini, "fopezen": fop, "mezinex": mez}
+    # Daborax at the same width and feed-forward: attention with the same heads, kv heads, key and value sizes and window as
+    # Fopezen's (a cap on the scores, learned sinks, no kept keys), linear attention with a decay per head in heads of the
+    # same size, and the state-space mixer of the Mezinex configuration; the fourth layer runs with the first one's tensors
+    dab_att = dict(heads=z["heads"], kv_heads=z["kv"], dim=z["dim"], vdim=z["vdim"], scale=z["dim"] ** -0.5, softcap=50.0,
+                   mask=dict(size=z["window"]))
+    dab_lin = dict(heads=z["heads"], dim=z["dim"], vdim=z["dim"], decay=[1.0 - 2.0 ** (-5 - 3 * h / z["heads"]) for h in range(z["heads"])])
+    dab_kinds = [("attention", dab_att), ("lightning", dab_lin), ("mamba2", ssm)]
+    dab_layers = []
+    for i in range(layers):
+        l = dict(type=dab_kinds[i % 4 % 3][0], mixer=dab_kinds[i % 4 % 3][1], mlp=dict(kind="dense", ff=z["ff"], limit=7.0))
+        if i % 4 == 3:
+            l["weights_of"] = i - 3
+        dab_layers.append(l)
+    dab = dict(architecture="Daborax", vocab=z["vocab"], width=z["width"], norm=dict(eps=1e-5), embedding=dict(scale=1.0),
+               residual_mult=0.5, layers=dab_layers)
+    return {"minicpm": mini, "fopezen": fop, "mezinex": mez, "daborax": dab}
 
 
 def _design_numbers(design, z, layers, kinds=None):
@@ -222,6 +237,8 @@ def _design_numbers(design, z, layers, kinds=None):
     eb = _elem_bytes()
     if design == "mezinex":
         return _mezinex_numbers(z, layers)
+    if design == "daborax":
+        return _daborax_numbers(z, layers)
     if design == "minicpm":
         per_layer = (H + 2 * G) * dk * d + H * dk * d + 3 * d * ff
         kv = lambda n: 2 * layers * G * dk * eb * n
@@ -268,6 +285,37 @@ def _mezinex_numbers(z, layers):
         per_tok_lin += 2.0 * n
     kv = lambda n: cache_row * n + state_bytes
     flops = lambda T: T * (per_tok_lin + scan) + sum(2.0 * w for w in walk) * (T * (T + 1) / 2) + 2.0 * V * d
+    return eb * weights, kv, flops
+
+
+def _daborax_numbers(z, layers):
+    """As ``_design_numbers`` for the Daborax configuration of ``_design_configs``.  A layer that runs with another's tensors
+    reads them again (they are counted per run: at these sizes a layer's matrices do not stay in the caches)."""
+    cfg = _design_configs(z, layers)["daborax"]
+    d, V, eb = z["width"], z["vocab"], _elem_bytes()
+    weights, per_tok_lin, scan, state_bytes = V * d, 0.0, 0.0, 0.0
+    spans = []         # (heads * (key + value size), kv heads * (key + value size), window) per attention layer
+    for l in cfg["layers"]:
+        m = l["mixer"]
+        n = 3 * d * l["mlp"]["ff"]
+        if l["type"] == "attention":
+            H, G, dk, dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+            n += (H * dk + G * dk + G * dv) * d + d * H * dv
+            spans.append((H * (dk + dv), G * (dk + dv), m["mask"]["size"]))
+        elif l["type"] == "lightning":
+            H, dk, dv = m["heads"], m["dim"], m["vdim"]
+            n += (2 * H * dk + 2 * H * dv) * d + d * H * dv
+            state_bytes += 2 * 4 * H * dk * dv
+            scan += 6.0 * H * dk * dv
+        else:
+            inner, gn = m["heads"] * m["vdim"], m["groups"] * m["state"]
+            n += (2 * inner + 2 * gn + m["heads"]) * d + d * inner
+            state_bytes += 2 * 4 * (inner * m["state"] + (m["conv"] - 1) * (inner + 2 * gn))
+            scan += 6.0 * inner * m["state"]
+        weights += n
+        per_tok_lin += 2.0 * n
+    kv = lambda n: sum(g * eb * min(n, w) for _, g, w in spans) + state_bytes
+    flops = lambda T: T * (per_tok_lin + scan) + sum(2.0 * h * sum(min(i + 1, w) for i in range(T)) for h, _, w in spans) + 2.0 * V * d
     return eb * weights, kv, flops
 
 
@@ -406,7 +454,7 @@ def main():
     ap.add_argument("--layers", type=int, default=0, help="fewer layers than the shape has (0: all)")
     ap.add_argument("--shape", default=None, choices=sorted(SHAPES), help="2b is the benchmark's configuration (default; 1b for --workload mixed)")
     ap.add_argument("--sizes", default=None, help="--workload designs: comma-separated sizes (default: all of 2b-like, 8b-like, 1b-like)")
-    ap.add_argument("--only", default=None, choices=["fopezen", "minicpm", "mezinex"], help="--workload designs: one design only")
+    ap.add_argument("--only", default=None, choices=["fopezen", "minicpm", "mezinex", "daborax"], help="--workload designs: one design only")
     ap.add_argument("--workload", default="decode", choices=["decode", "mixed", "long", "designs"],
                     help="decode: the benchmark (prefill of one prompt, decode steps at fixed batches); "
                          "mixed: 64 requests of 128..2048 prompt tokens through the scheduler, --steps tokens generated each; "
