@@ -58,6 +58,13 @@ __device__ __forceinline__ float silu_mul_fast(float g, float u) {
     return u * g * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * g));
 }
 
+// The gated unit with bounded branches: g = min(gate, limit), u = clamp(up, -limit, limit), g sigmoid(slope g) (u + 1).
+__device__ __forceinline__ float glu_clamped_f(float g, float u, float limit, float slope) {
+    g = fminf(g, limit);
+    u = fminf(fmaxf(u, -limit), limit);
+    return g / (1.0f + expf(-slope * g)) * (u + 1.0f);
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);

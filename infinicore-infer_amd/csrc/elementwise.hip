@@ -296,9 +296,7 @@ __global__ void glu_clamped_kernel(const T* __restrict__ gu, T* __restrict__ out
     for (; i < n; i += step) {
         const size_t t = i / di;
         const int j = (int)(i - t * di);
-        const float g = fminf(to_f32(gu[t * 2 * (size_t)di + j]), limit);
-        const float u = fminf(fmaxf(to_f32(gu[t * 2 * (size_t)di + di + j]), -limit), limit);
-        out[i] = from_f32<T>(g / (1.0f + expf(-alpha * g)) * (u + 1.0f));
+        out[i] = from_f32<T>(glu_clamped_f(to_f32(gu[t * 2 * (size_t)di + j]), to_f32(gu[t * 2 * (size_t)di + di + j]), limit, alpha));
     }
 }
 
@@ -315,10 +313,7 @@ __global__ void glu_clamped_vec8_kernel(const bf16* __restrict__ gu, bf16* __res
         load4(gp, g); load4(gp + 4, g + 4);
         load4(gp + di, u); load4(gp + di + 4, u + 4);
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            const float gg = fminf(g[e], limit), uu = fminf(fmaxf(u[e], -limit), limit);
-            o[e] = gg / (1.0f + expf(-alpha * gg)) * (uu + 1.0f);
-        }
+        for (int e = 0; e < 8; ++e) o[e] = glu_clamped_f(g[e], u[e], limit, alpha);
         bf16* op = out + t * (size_t)di + j;
         store4(op, o); store4(op + 4, o + 4);
     }

@@ -75,6 +75,7 @@ struct NormFuse {
     float* ss_out;             // [gridDim.x, 16]
     int act;                   // plain store only: 0 none, else the product (rounded to its type first, as when stored) goes
                                // through an activation: 1 relu(z)^2, 2 gelu_tanh(z), 3 silu(z)
+    float glu_limit, glu_slope; // the gated epilogue: limit > 0: the unit with bounded branches instead of up * silu(gate)
 };
 
 __device__ __forceinline__ float gemm_act(float z, int act) {
@@ -376,7 +377,8 @@ gemm_nt_bf16_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__
                     g = to_f32(from_f32<TC>(alpha * g));
                     u = to_f32(from_f32<TC>(alpha * u));
                     const int n = n0 + 16 * gi + 4 * kq + e;
-                    if (m < M && n < sw_end) C[(size_t)m * ldc + n] = from_f32<TC>(silu_mul_fast(g, u));
+                    if (m < M && n < sw_end)
+                        C[(size_t)m * ldc + n] = from_f32<TC>(nf.glu_limit > 0.f ? glu_clamped_f(g, u, nf.glu_limit, nf.glu_slope) : silu_mul_fast(g, u));
                 }
         }
         return;
@@ -881,9 +883,28 @@ IC_EXPORT int ic_gemm_nt_residual_parts(int N) {
 // c_mode 2 (M <= 16, bfloat16 C, `tail` given): x += tail->alpha * (alpha * A W^T); C = x * tail->weight;
 // tail->sumsq_out[b * 16 + m] = sum of x[m]^2 over column block b.  row_factor (M <= 16, any c_mode): row m
 // of the product is multiplied by rsqrt(sum_b sumsq[b * 16 + m] / width + eps) first.
+// ic_gemm_nt_glu_clamped: c_mode 1 with the gated unit of bounded branches in place of SwiGLU,
+// C [M, N/2] = g sigmoid(slope g) (u + 1), g = min(gate, limit), u = clamp(up, -limit, limit).
+static int gemm_nt_impl(const void* A, int a_dtype, const void* W, int w_dtype, void* C, int c_dtype,
+                        int M, int N, int K, int lda, int ldw, int ldc, float alpha, int c_mode,
+                        const IcRowFactor* row_factor, const IcResidualNorm* tail, float glu_limit, float glu_slope, hipStream_t stream);
+
 IC_EXPORT int ic_gemm_nt(const void* A, int a_dtype, const void* W, int w_dtype, void* C, int c_dtype,
                          int M, int N, int K, int lda, int ldw, int ldc, float alpha, int c_mode,
                          const IcRowFactor* row_factor, const IcResidualNorm* tail, hipStream_t stream) {
+    return gemm_nt_impl(A, a_dtype, W, w_dtype, C, c_dtype, M, N, K, lda, ldw, ldc, alpha, c_mode, row_factor, tail, 0.f, 0.f, stream);
+}
+
+IC_EXPORT int ic_gemm_nt_glu_clamped(const void* A, int a_dtype, const void* W, int w_dtype, void* C, int c_dtype,
+                                     int M, int N, int K, int lda, int ldw, int ldc, float limit, float slope,
+                                     const IcRowFactor* row_factor, hipStream_t stream) {
+    if (!(limit > 0.f)) return IC_ERR_ARG;
+    return gemm_nt_impl(A, a_dtype, W, w_dtype, C, c_dtype, M, N, K, lda, ldw, ldc, 1.0f, 1, row_factor, nullptr, limit, slope, stream);
+}
+
+static int gemm_nt_impl(const void* A, int a_dtype, const void* W, int w_dtype, void* C, int c_dtype,
+                        int M, int N, int K, int lda, int ldw, int ldc, float alpha, int c_mode,
+                        const IcRowFactor* row_factor, const IcResidualNorm* tail, float glu_limit, float glu_slope, hipStream_t stream) {
     if (M <= 0 || N <= 0) return IC_OK;
     if (K <= 0 || lda < K || ldw < K || c_mode < 0 || c_mode > 5) return IC_ERR_ARG;
     if (c_mode == 1 ? ((N & 1) || ldc < N / 2) : (ldc < N)) return IC_ERR_ARG;
@@ -892,6 +913,8 @@ IC_EXPORT int ic_gemm_nt(const void* A, int a_dtype, const void* W, int w_dtype,
     if ((M + 63) / 64 > 65535) return IC_ERR_ARG;
     NormFuse nf{};
     if (c_mode >= 3) { nf.act = c_mode - 2; c_mode = 0; }      // the plain product with an activation on its way out
+    nf.glu_limit = glu_limit;
+    nf.glu_slope = glu_slope;
     if (!norm_fuse_args(row_factor, tail, M, N, K, c_dtype, ic_gemm_nt_residual_parts(N), nf)) return IC_ERR_ARG;
     const bool aligned = (lda % 8 == 0) && (ldw % 8 == 0) && (((uintptr_t)A & 15) == 0) && (((uintptr_t)W & 15) == 0);
     if (c_mode == 1 && M > 16 && (M > 32 || c_dtype != IC_BF16 || row_factor || !lines_apply(aligned, K))) return IC_ERR_ARG;

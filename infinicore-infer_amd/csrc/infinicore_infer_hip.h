@@ -119,6 +119,8 @@ typedef struct {
 int ic_gemm_nt_supported(int a_dtype, int w_dtype, int c_dtype);
 int ic_gemm_nt_residual_parts(int N);
 int ic_gemm_nt(const void* A, int a_dtype, const void* W, int w_dtype, void* C, int c_dtype, int M, int N, int K, int lda, int ldw, int ldc, float alpha, int c_mode, const IcRowFactor* row_factor, const IcResidualNorm* tail, hipStream_t stream);
+// As c_mode 1 with W = [gate; up] and C [M, N/2] = g sigmoid(slope g) (u + 1), g = min(gate, limit), u = clamp(up, -limit, limit).
+int ic_gemm_nt_glu_clamped(const void* A, int a_dtype, const void* W, int w_dtype, void* C, int c_dtype, int M, int N, int K, int lda, int ldw, int ldc, float limit, float slope, const IcRowFactor* row_factor, hipStream_t stream);
 // Rows that the products with an epilogue take: kind 1 (c_mode 1, SwiGLU) and kind 2 (ic_gemm_qkv_rope) 32 where the weights can be
 // read in whole cache lines (K a multiple of 64, row strides multiples of 8), 16 otherwise; without row factors above 16 rows.
 int ic_gemm_nt_epilogue_rows(int kind, int K, int lda, int ldw);

@@ -138,6 +138,7 @@ _SIGNATURES = {
     "ic_argmax_static_max_rows": [],
     "ic_argmax_static": [_P, _LL, _I, _I, _P, _P],
     "ic_gemm_nt": [_P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _F, _I, _RF, _RN, _P],
+    "ic_gemm_nt_glu_clamped": [_P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _F, _F, _RF, _P],
     "ic_gemm_nt_residual_parts": [_I],
     "ic_gemm_nt_variant": [_P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _F, _I, _RF, _RN, _I, _P],
     "ic_gemm_nt_epilogue_rows": [_I, _I, _I, _I],

@@ -450,7 +450,7 @@ def gemm_epilogue_rows(kind: str, a, w) -> int:
 
 
 def gemm_nt(a, w, out, alpha: float = 1.0, swiglu_output: bool = False, row_factor=None, residual=None, whole_lines: bool = True,
-            activation=None):
+            activation=None, glu_clamped=None):
     """out[M, N] = alpha * a[M, K] @ w[N, K]^T (bfloat16 operands, float32 accumulation).
     swiglu_output (M <= gemm_epilogue_rows("swiglu", a, w)): w = [gate rows; up rows] and out[M, N/2] = up * silu(gate).
     row_factor = (sumsq [n_parts, 16], width, eps), M <= 16: row m of the product is first multiplied by
@@ -459,7 +459,8 @@ def gemm_nt(a, w, out, alpha: float = 1.0, swiglu_output: bool = False, row_fact
     M <= 16, bfloat16 out: x += beta * (the product rounded to bfloat16); out = x * weight;
     sumsq_out[b, m] = sum of x[m]^2 over columns 16 b .. 16 b + 15.
     whole_lines False (tests): the weights are loaded in operand layout also where whole cache lines would apply.
-    activation ("relu2", "gelu_tanh", "silu"; not with the other epilogues): out = act(the product as rounded to out's dtype)."""
+    activation ("relu2", "gelu_tanh", "silu"; not with the other epilogues): out = act(the product as rounded to out's dtype).
+    glu_clamped = (limit, slope), with swiglu_output: out = g sigmoid(slope g) (u + 1), g = min(gate, limit), u = clamp(up, -limit, limit)."""
     import ctypes
     _dev(a, w, out)
     M, K = a.shape
@@ -484,6 +485,13 @@ def gemm_nt(a, w, out, alpha: float = 1.0, swiglu_output: bool = False, row_fact
     if activation is not None:
         _need(mode == 0 and activation in ACTIVATIONS, "gemm_nt: an activation goes with the plain product only (have %s)" % ", ".join(sorted(ACTIVATIONS)))
         mode = 3 + ACTIVATIONS[activation]
+    if glu_clamped is not None:
+        _need(swiglu_output and whole_lines and alpha == 1.0, "gemm_nt: the bounded gated unit is an epilogue of the gate/up product")
+        check(get_lib().ic_gemm_nt_glu_clamped(a.data_ptr(), dtype_code(a.dtype), w.data_ptr(), dtype_code(w.dtype),
+                                               out.data_ptr(), dtype_code(out.dtype), M, N, K, a.stride(0), w.stride(0),
+                                               out.stride(0), float(glu_clamped[0]), float(glu_clamped[1]),
+                                               ctypes.byref(rf) if rf else None, _stream()), "gemm_nt")
+        return out
     if not whole_lines:
         check(get_lib().ic_gemm_nt_variant(a.data_ptr(), dtype_code(a.dtype), w.data_ptr(), dtype_code(w.dtype),
                                            out.data_ptr(), dtype_code(out.dtype), M, N, K, a.stride(0), w.stride(0),

@@ -73,14 +73,15 @@ class SwiGLU(FeedForward):
         act = ctx.ws.buffer("ffn_act", (T, self.intermediate_size), rt.dtype)
         owed = isinstance(h, DeferredRows)
         rows = h.values if owed else h
-        few = (self.variant == "silu" and rt.gemm_impl == "auto" and rows.dtype == self.w_gate_up.dtype == act.dtype
+        few = (rt.gemm_impl == "auto" and rows.dtype == self.w_gate_up.dtype == act.dtype
                and ops.rule_gate_up_fused(rows.dtype, T, rows, self.w_gate_up, owed))
         if few:
             # few rows: the activation is the epilogue of the gate/up projection
+            unit = (self.limit, self.alpha) if self.variant == "clamped" else None
             if isinstance(h, DeferredRows):
-                ops.gemm_nt(h.values, self.w_gate_up, act, swiglu_output=True, row_factor=h.row_factor())
+                ops.gemm_nt(h.values, self.w_gate_up, act, swiglu_output=True, row_factor=h.row_factor(), glu_clamped=unit)
             else:
-                ops.gemm_nt(h, self.w_gate_up, act, swiglu_output=True)
+                ops.gemm_nt(h, self.w_gate_up, act, swiglu_output=True, glu_clamped=unit)
         else:
             gate_up = ctx.ws.buffer("gate_up", (T, 2 * self.intermediate_size), rt.dtype)
             linear(h, self.w_gate_up, gate_up, rt.gemm_impl, ws=ctx.ws)

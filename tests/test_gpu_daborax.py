@@ -274,6 +274,26 @@ def test_clamped_gated_unit(dtype):
     assert torch.allclose(odd.cpu().double(), want[:, :di - 1], atol=1e-5 if dtype == torch.float32 else 2e-2)
 
 
+@pytest.mark.parametrize("M,K,di", [(1, 96, 40), (8, 256, 128), (16, 200, 72), (3, 4096, 1024), (24, 512, 256), (32, 1024, 512)])
+def test_bounded_gated_unit_as_the_epilogue_of_the_gate_up_product(M, K, di):
+    """Few rows: the unit rides in the product's epilogue (both projections rounded to bfloat16 first, as when stored)."""
+    from infinicore_infer_amd.kernels import ops
+    limit, slope = 1.2, 1.702
+    g = torch.Generator().manual_seed(M + di)
+    a = torch.randn(M, K, generator=g).to(torch.bfloat16)
+    w = (2.5 * torch.randn(2 * di, K, generator=g) / math.sqrt(K)).to(torch.bfloat16)
+    if not ops.rule_gate_up_fused(torch.bfloat16, M, _dev(a), _dev(w), False):
+        assert M > 16
+        pytest.skip("these operands take the library product and the unit's own kernel")
+    gu = (a.double() @ w.double().T).to(torch.bfloat16).double()
+    gt, up = torch.clamp(gu[:, :di], max=limit), torch.clamp(gu[:, di:], -limit, limit)
+    want = gt * torch.sigmoid(slope * gt) * (up + 1)
+    assert float((gu[:, :di] > limit).double().mean()) > 0.02 and float((gu[:, di:].abs() > limit).double().mean()) > 0.05
+    out = torch.empty(M, di, dtype=torch.bfloat16, device="cuda")
+    ops.gemm_nt(_dev(a), _dev(w), out, swiglu_output=True, glu_clamped=(limit, slope))
+    assert torch.allclose(out.cpu().double(), want, atol=3e-2, rtol=2e-2)
+
+
 def test_norm_then_weight_then_sigmoid_gate():
     from infinicore_infer_amd.kernels import ops
     T, n, eps = 5, 60, 1e-5
