@@ -138,6 +138,86 @@ def test_replay_modes(tmp_path_factory, name, dname, dtype, tol, mode):
         assert engine.cache.free_pages(g) == engine.num_pages
 
 
+def _misread(monkeypatch, what):
+    """One plausible misreading put into the plain implementation."""
+    if what == "window one token longer":
+        real = P.seen
+        monkeypatch.setattr(P, "seen", lambda n, k, window, first=0: real(n, k, None if window is None else window + 1, first))
+    elif what == "window one token shorter":
+        real = P.seen
+        monkeypatch.setattr(P, "seen", lambda n, k, window, first=0: real(n, k, None if window is None else window - 1, first))
+    elif what == "no sink":
+        real = P.sink_softmax
+        monkeypatch.setattr(P, "sink_softmax", lambda s, m, sink, softcap=None: real(s, m, None, softcap))
+    elif what == "sink capped and scaled away to zero":
+        real = P.sink_softmax
+        monkeypatch.setattr(P, "sink_softmax", lambda s, m, sink, softcap=None: real(s, m, 0.0 * sink, softcap))
+    elif what == "no cap":
+        real = P.sink_softmax
+        monkeypatch.setattr(P, "sink_softmax", lambda s, m, sink, softcap=None: real(s, m, sink, None))
+    elif what == "query head h on kv head h % kv_heads":
+        real = P.window_attention
+
+        def rolled(h, W, p, heads, kv_heads, dim, vdim, scale, softcap, window, eps):
+            W = dict(W)
+            order = [hd % kv_heads * (heads // kv_heads) + hd // kv_heads for hd in range(heads)]      # (a permutation of the heads)
+            W[p + "q"] = W[p + "q"].view(heads, dim, -1)[order].reshape(heads * dim, -1)
+            return real(h, W, p, heads, kv_heads, dim, vdim, scale, softcap, window, eps)
+        monkeypatch.setattr(P, "window_attention", rolled)
+    elif what == "decays of the heads in reverse":
+        real = P.lightning_mixer
+        monkeypatch.setattr(P, "lightning_mixer", lambda h, W, p, heads, dim, vdim, decay, eps: real(h, W, p, heads, dim, vdim, decay[::-1], eps))
+    elif what == "the new key decays too":
+        def late(h, W, p, heads, dim, vdim, decay, eps):
+            T = h.shape[0]
+            q, k = (P.silu(h @ W[p + n].T).reshape(T, heads, dim) for n in "qk")
+            v = P.silu(h @ W[p + "v"].T).reshape(T, heads, vdim)
+            o = torch.zeros(T, heads, vdim, dtype=h.dtype)
+            for hd in range(heads):
+                S = torch.zeros(dim, vdim, dtype=h.dtype)
+                for t in range(T):
+                    S = decay[hd] * (S + torch.outer(k[t, hd], v[t, hd]))
+                    o[t, hd] = S.T @ q[t, hd]
+            o = P.unit_rms(o.reshape(T, heads * vdim), eps) * W[p + "norm"] * torch.sigmoid(h @ W[p + "g"].T)
+            return o @ W[p + "o"].T
+        monkeypatch.setattr(P, "lightning_mixer", late)
+    elif what == "layer scale left out":
+        real = P.forward
+
+        def unscaled(cfg, W, tokens, dtype=torch.float64, layers_out=None):
+            return real(cfg, {k: (torch.ones_like(v) if k.endswith((".ls1", ".ls2")) else v) for k, v in W.items()}, tokens, dtype, layers_out)
+        monkeypatch.setattr(P, "forward", unscaled)
+    elif what == "up branch not clamped":
+        def loose(h, W, p, limit):
+            g = torch.clamp(h @ W[p + "gate"].T, max=limit)
+            return (g * torch.sigmoid(1.702 * g) * (h @ W[p + "up"].T + 1.0)) @ W[p + "down"].T
+        monkeypatch.setattr(P, "clamped_glu", loose)
+    elif what == "two borrowing layers in the other order":
+        real = P.forward
+        monkeypatch.setattr(P, "forward", lambda cfg, W, tokens, dtype=torch.float64, layers_out=None: real(
+            dict(cfg, layers=cfg["layers"][:3] + [cfg["layers"][4], cfg["layers"][3]] + cfg["layers"][5:]), W, tokens, dtype, layers_out))
+    else:
+        raise ValueError(what)
+
+
+@pytest.mark.parametrize("what", ["window one token longer", "window one token shorter", "no sink", "sink capped and scaled away to zero",
+                                  "no cap", "query head h on kv head h % kv_heads", "decays of the heads in reverse",
+                                  "the new key decays too", "layer scale left out", "up branch not clamped",
+                                  "two borrowing layers in the other order"])
+def test_a_misreading_of_the_design_shows(tmp_path_factory, monkeypatch, what):
+    """The comparison the other tests rest on is sharp enough: with one misreading in the plain implementation the float32
+    engine no longer agrees with it (the same request agrees without)."""
+    folder, W = _model(tmp_path_factory, "D1")
+    toks = H.random_tokens(D1["vocab"], 120, 21)
+    engine = _engine(tmp_path_factory, "D1", torch.float32, 128)
+    steps, _ = H.trace_whole({"a": toks})
+    got = H.run_trace(engine, steps)
+    H.compare(got, {"a": P.forward(D1, W, toks, torch.float64)}, 2e-4, "as designed")
+    _misread(monkeypatch, what)
+    with pytest.raises(AssertionError):
+        H.compare(got, {"a": P.forward(D1, W, toks, torch.float64)}, 2e-4, what)
+
+
 def test_the_residual_stream_after_every_layer(tmp_path_factory):
     """Layer by layer in float32, a layer that runs twice counted each time: the stream after every entry of the run order."""
     from infinicore_infer_amd.engine import Engine, StepEntry
