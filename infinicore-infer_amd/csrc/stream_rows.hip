@@ -49,7 +49,10 @@ template <int N> __device__ __forceinline__ void load_floats(const float* p, flo
 
 // ---------------------------------------------------------------------------------------------
 // x[t, 2i] = table[tok, 2i] * scale + sin(p f_i), x[t, 2i+1] = table[tok, 2i+1] * scale + cos(p f_i);
-// f_i is a float32 table [ceil(d/2)] made by the host; the angle is the float32 product p * f_i.
+// f_i comes as two float32 tables of n = ceil(d/2) entries made by the host from the float64 value: freq[i] its
+// rounding and freq[n + i] what the rounding left.  The angle is the float32 product p * freq[i] plus a small
+// rest (the product's own rounding error, from an fma, and p * freq[n + i]); sine and cosine of the sum follow
+// from those of the product to second order in the rest, so that far positions keep float32 accuracy.
 // copy (nullable): x rounded to the compute dtype.
 // ---------------------------------------------------------------------------------------------
 template <typename TW, typename TC>
@@ -60,13 +63,17 @@ __global__ void embed_sinusoid_kernel(const int* __restrict__ tokens, const int*
     const TW* row = table + (size_t)tokens[t] * d;
     const float p = (float)positions[t];
     float* o = x + (size_t)t * d;
-    for (int i = threadIdx.x; i < (d + 1) / 2; i += blockDim.x) {
-        const float ang = p * freq[i];
-        const float a = to_f32(row[2 * i]) * scale + sinf(ang);
+    const int n = (d + 1) / 2;
+    for (int i = threadIdx.x; i < n; i += blockDim.x) {
+        const float f = freq[i];
+        const float ang = p * f;
+        const float rest = fmaf(p, f, -ang) + p * freq[n + i];
+        const float sn = sinf(ang), cs = cosf(ang), half = 0.5f * rest * rest;
+        const float a = to_f32(row[2 * i]) * scale + ((sn - half * sn) + rest * cs);
         o[2 * i] = a;
         if (copy) copy[(size_t)t * d + 2 * i] = from_f32<TC>(a);
         if (2 * i + 1 < d) {                              // an odd width ends on a sine
-            const float b = to_f32(row[2 * i + 1]) * scale + cosf(ang);
+            const float b = to_f32(row[2 * i + 1]) * scale + ((cs - half * cs) - rest * sn);
             o[2 * i + 1] = b;
             if (copy) copy[(size_t)t * d + 2 * i + 1] = from_f32<TC>(b);
         }

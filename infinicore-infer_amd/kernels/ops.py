@@ -682,7 +682,8 @@ ACTIVATIONS = {"relu2": 0, "gelu_tanh": 1, "silu": 2}
 
 
 def embed_sinusoid(tokens, positions, table, freq, out, copy=None, scale: float = 1.0):
-    """out[t, 2i] = table[tokens[t], 2i] * scale + sin(positions[t] * freq[i]), out[t, 2i+1] = .. + cos(..);
+    """out[t, 2i] = table[tokens[t], 2i] * scale + sin(positions[t] * f_i), out[t, 2i+1] = .. + cos(..);
+    ``freq`` is float32 [2, ceil(d/2)]: f_i rounded, and what the rounding left (zeros: the rounded value alone).
     out is float32 [T, d]; ``copy`` (optional, [T, d]) receives out rounded to its dtype."""
     _dev(tokens, positions, table, freq, out, copy)
     _i32(tokens, "tokens")
@@ -691,7 +692,8 @@ def embed_sinusoid(tokens, positions, table, freq, out, copy=None, scale: float 
     _need(tokens.numel() == T and positions.numel() == T and table.dim() == 2 and table.shape[1] == d,
           "embed_sinusoid: shape mismatch")
     _need(out.dtype == torch.float32 and out.is_contiguous() and table.is_contiguous(), "embed_sinusoid: layout")
-    _need(freq.dtype == torch.float32 and freq.is_contiguous() and freq.numel() == (d + 1) // 2, "embed_sinusoid: freq must be float32 [ceil(d/2)]")
+    _need(freq.dtype == torch.float32 and freq.is_contiguous() and tuple(freq.shape) == (2, (d + 1) // 2),
+          "embed_sinusoid: freq must be float32 [2, ceil(d/2)]")
     if copy is not None:
         _need(tuple(copy.shape) == (T, d) and copy.is_contiguous(), "embed_sinusoid: copy layout")
     check(get_lib().ic_embed_sinusoid(tokens.data_ptr(), positions.data_ptr(), table.data_ptr(), dtype_code(table.dtype),

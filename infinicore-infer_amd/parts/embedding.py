@@ -17,10 +17,13 @@ from .linear import linear
 
 
 def sinusoid_frequencies(width: int, base: float) -> torch.Tensor:
-    """f_i = base^(-2i/width) for 2i < width, in float32 arithmetic (the angle of position p is the float32
-    product p * f_i)."""
-    i = torch.arange((width + 1) // 2, dtype=torch.float32)
-    return torch.pow(torch.tensor(base, dtype=torch.float32), -2.0 * i / width).contiguous()
+    """f_i = base^(-2i/width) for 2i < width as float32 [2, ceil(width/2)]: row 0 the float64 value rounded, row 1
+    what the rounding left.  The kernel forms the angle of position p from both, so that its error does not grow
+    with p."""
+    i = torch.arange((width + 1) // 2, dtype=torch.float64)
+    f = torch.pow(torch.tensor(base, dtype=torch.float64), -2.0 * i / width)
+    hi = f.to(torch.float32)
+    return torch.stack([hi, (f - hi.double()).to(torch.float32)]).contiguous()
 
 
 @register_part("embedding", "embedding")

@@ -169,16 +169,14 @@ def test_embedding_with_position_vector(width, first):
     table = torch.randn(50, width, generator=g).to(torch.bfloat16)
     tokens = torch.randint(0, 50, (37,), generator=g)
     pos = torch.arange(first, first + 37)
-    want = table.float()[tokens] + P.sinusoid(pos, width, torch.float32)
     x = torch.empty(37, width, dtype=torch.float32, device="cuda")
     copy = torch.empty(37, width, dtype=torch.bfloat16, device="cuda")
     ops.embed_sinusoid(_dev(tokens, torch.int32), _dev(pos, torch.int32), _dev(table), sinusoid_frequencies(width, 10000.0).cuda(),
                        x, copy=copy)
-    # float32 angles of large positions: the kernel and torch may round sin/cos differently in the last place
-    assert float((x.cpu() - want).abs().max()) < 2e-6 * max(1.0, 1.0)
     assert torch.equal(copy.cpu(), x.cpu().to(torch.bfloat16))
+    # far positions too: the angle keeps what the float32 product p * f rounds away
     exact = table.double()[tokens] + P.sinusoid(pos, width, torch.float64)
-    assert float((x.cpu().double() - exact).abs().max()) < 1e-2 if first > 10000 else float((x.cpu().double() - exact).abs().max()) < 1e-4
+    assert float((x.cpu().double() - exact).abs().max()) < 2e-6
 
 
 @pytest.mark.parametrize("d,bias", [(64, False), (200, True), (1026, True)])
