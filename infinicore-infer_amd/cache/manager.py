@@ -39,8 +39,11 @@ class GroupSpec:
     planes: int = 2                     # tensors per slot (keys and values: 2; one latent per token: 1)
     plane_dims: tuple = ()              # width of each plane when they differ; empty: all head_dim
     keep_first: int = 0                 # 'window': the first tokens that stay readable for good
+    stride: int = 1                     # tokens per row: a group with stride P holds one row for every COMPLETE block of P tokens
 
     def __post_init__(self):
+        if self.stride < 1 or (self.stride > 1 and self.kind != "full"):
+            raise CacheError("a group's stride is a positive token count, and a strided group keeps every row")
         if self.kind not in ("full", "window"):
             raise CacheError("group kind must be 'full' or 'window'")
         if self.kind == "window" and not (self.window and self.window > 0):
@@ -139,14 +142,20 @@ class CacheManager:
         return slot
 
     # ---- growth ---------------------------------------------------------------
-    def _pages_for(self, length: int) -> int:
-        return (length + self.page_size - 1) // self.page_size
+    def _pages_for(self, length: int, group: Optional[int] = None) -> int:
+        """Pages that hold the rows of ``length`` tokens: one row a token, or in a strided group one row for every
+        complete block of ``stride`` tokens."""
+        rows = length if group is None else length // self.groups[group].stride
+        return (rows + self.page_size - 1) // self.page_size
+
+    def pages_for_tokens(self, length: int) -> List[int]:
+        """Pages per group that a request of ``length`` tokens holds."""
+        return [self._pages_for(length, g) for g in range(len(self.groups))]
 
     def pages_needed(self, req_id, n_new: int) -> List[int]:
         """New pages per group that appending n_new tokens would take."""
         e = self.requests[req_id]
-        want = self._pages_for(e.length + n_new)
-        return [max(0, want - len(t)) for t in e.tables]
+        return [max(0, self._pages_for(e.length + n_new, g) - len(t)) for g, t in enumerate(e.tables)]
 
     def can_append(self, req_id, n_new: int, reserve: Optional[List[int]] = None) -> bool:
         """True when the pools hold the pages for n_new more tokens, beyond
@@ -184,8 +193,8 @@ class CacheManager:
         e = self.requests[req_id]
         if length > e.length or length < 0:
             raise CacheError("truncate: request %r holds %d tokens, %d asked" % (req_id, e.length, length))
-        keep = self._pages_for(length)
         for g, table in enumerate(e.tables):
+            keep = self._pages_for(length, g)
             while len(table) > keep:
                 p = table.pop()
                 if p >= 0:
@@ -216,8 +225,8 @@ class CacheManager:
             raise CacheError("request %r is already admitted" % (dst_id,))
         if self.slots.n_free == 0:
             raise OutOfPages("no free state slot (max_requests = %d)" % self.max_requests)
-        n_pages = self._pages_for(n)
-        live = [[j for j in range(min(n_pages, len(t))) if t[j] >= 0] for t in src.tables]
+        n_pages_of = self.pages_for_tokens(n)
+        live = [[j for j in range(min(n_pages_of[g], len(t))) if t[j] >= 0] for g, t in enumerate(src.tables)]
         for g, idx in enumerate(live):
             if len(idx) > self.pools[g].n_free:
                 raise OutOfPages("fork needs %d pages of group %d, %d free" % (len(idx), g, self.pools[g].n_free))
@@ -225,6 +234,7 @@ class CacheManager:
         dst = self.requests[dst_id]
         pairs = []
         for g, idx in enumerate(live):
+            n_pages = n_pages_of[g]
             table = [-1] * n_pages                # pages the source gave back (behind a window) stay given back
             for j in idx:
                 table[j] = self.pools[g].alloc()
@@ -274,7 +284,7 @@ class CacheManager:
         return self.requests[req_id].tables[group]
 
     def slot_of(self, req_id, group: int, position: int) -> int:
-        """Physical token slot (page * page_size + offset) of a position."""
+        """Physical token slot (page * page_size + offset) of a position (of a row, in a strided group)."""
         page = self.requests[req_id].tables[group][position // self.page_size]
         if page < 0:
             raise CacheError("position %d of request %r lies in a page that was given back" % (position, req_id))

@@ -24,6 +24,7 @@ class CacheStorage:
         self.device = device
         self.group_planes: List[torch.Tensor] = []
         self._slot_index: Dict[int, Tuple[int, int]] = {}      # cache slot -> (group, index in group)
+        self._strided_index: Dict[int, Tuple[int, int]] = {}   # cache slot -> (its strided group, index in it): rows per block of tokens
         for g, spec in enumerate(groups):
             dims = spec.dims()
             if len(set(dims)) == 1:
@@ -35,9 +36,9 @@ class CacheStorage:
                                            dtype=dtype, device=device) for w in dims)
             self.group_planes.append(planes)
             for i, s in enumerate(spec.slots):
-                self._slot_index[s] = (g, i)
+                (self._strided_index if spec.stride > 1 else self._slot_index)[s] = (g, i)
         self.state: Dict[int, torch.Tensor] = {}               # cache slot -> [max_requests, ...]
-        self._kv_views: Dict[int, tuple] = {}
+        self._kv_views: Dict[object, tuple] = {}
         self._copy_idx = None                                  # (pinned, device) page ids of copy_pages, kept between calls
 
     def add_state(self, slot: int, max_requests: int, shape, dtype) -> torch.Tensor:
@@ -60,6 +61,17 @@ class CacheStorage:
             else:
                 views = tuple(gp[i, j] for j in range(gp.shape[1]))
             self._kv_views[slot] = views
+        return views
+
+    def strided_planes(self, slot: int) -> tuple:
+        """The planes of a cache slot's strided group (one row per block of tokens), each [num_pages, n_kv_heads, page_size, width]."""
+        key = ("strided", slot)
+        views = self._kv_views.get(key)
+        if views is None:
+            g, i = self._strided_index[slot]
+            gp = self.group_planes[g]
+            views = tuple(p[i, 0] for p in gp) if isinstance(gp, tuple) else tuple(gp[i, j] for j in range(gp.shape[1]))
+            self._kv_views[key] = views
         return views
 
     def kv(self, slot: int):

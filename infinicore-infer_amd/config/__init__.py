@@ -6,10 +6,11 @@ from .minicpm import MiniCPMConfig, RopeScaling
 from .fopezen import FopezenConfig
 from .mezinex import MezinexConfig
 from .daborax import DaboraxConfig
+from .fizelix import FizelixConfig
 
 __all__ = [
     "ConfigError", "config_from_dict", "config_from_dir", "read_config_json",
     "register_architecture", "registered_architectures", "resolve_architecture",
     "ExecEntry", "LayerSpec", "ModelSpec", "PartSpec", "default_schedule",
-    "MiniCPMConfig", "RopeScaling", "FopezenConfig", "MezinexConfig", "DaboraxConfig",
+    "MiniCPMConfig", "RopeScaling", "FopezenConfig", "MezinexConfig", "DaboraxConfig", "FizelixConfig",
 ]

@@ -43,10 +43,14 @@ class ExecEntry:
                 every entry has a slot of its own.
     ``writes_cache``  False when the entry only reads a slot that an earlier
                 entry wrote (a layer reading another layer's cache).
+    ``adds_embedding``  True when the embedding's output (the residual stream as it
+                was before the first entry) is added to the stream right before
+                this entry runs: the first layer of a repeated pass.
     """
     layer: int
     cache: int
     writes_cache: bool = True
+    adds_embedding: bool = False
 
 
 @dataclass(frozen=True)

@@ -150,6 +150,26 @@ int ic_matmul(const void* A, int a_dtype, const void* W, void* C, int c_dtype, i
 // flush (or nullptr): memory larger than the caches, overwritten before every timed launch so that operands come from memory.
 int ic_matmul_tune(const void* A, int a_dtype, const void* W, void* C, int c_dtype, int M, int N, int K, int lda, int ldw, int ldc, void* workspace, long long workspace_bytes, void* flush, long long flush_bytes, int reps, hipStream_t stream);
 
+// ---- attn_pooled.hip: a window of tokens plus one mean key/value per block before it, sigmoid weights ---------------
+// Adjacent pairs (2i, 2i+1) of the first rot_dims entries of every q and k head turn by position * f_i (freq: float32
+// [2, rot_dims / 2], the rounded frequency and what the rounding left); q -> q_out, k and v -> the cache at slots (null: q only).
+int ic_rope_pairs_store(const void* rows, int row_stride, int dtype, const int* positions, const float* freq, int rot_dims, void* q_out, void* kcache, void* vcache, const int* slots, int T, int nh, int nkvh, int dk, int dv, int page_size, hipStream_t stream);
+// Means of the blocks of P tokens that the step's tokens complete, from the token cache into row b of the block-mean cache.
+int ic_pool_blocks(const void* kcache, const void* vcache, void* kpool, void* vpool, int dtype, const int* block_tables, int bt_stride, const int* pool_tables, int pt_stride, const int* token_req, const int* positions, int T, int P, int nkvh, int dk, int dv, int page_size, hipStream_t stream);
+// out_i = sum over seen tokens and blocks of sigmoid(scale q.k + bias[h]) v; any sizes up to 512, float32 or bfloat16.
+int ic_attn_pooled_generic(const void* q, int q_stride, void* out, int out_stride, int dtype, const void* kcache, const void* vcache, const void* kpool, const void* vpool, const int* block_tables, int bt_stride, const int* pool_tables, int pt_stride, const int* token_req, const int* positions, const float* bias, int T, int nh, int nkvh, int dk, int dv, int page_size, float scale, int window, int P, hipStream_t stream);
+
+// ---- moe.hip: routed experts --------------------------------------------------------------------------------------
+int ic_moe_route(const float* z, int z_stride, int T, int E, int top, int mode, int renorm, int* ids, float* weights, hipStream_t stream);
+int ic_moe_sort(const int* ids, int n, int E, int* offsets, int* order, int* place, hipStream_t stream);
+int ic_moe_gather(const void* h, int h_stride, int dtype, const int* order, const float* weights, int n, int top, int d, void* out, hipStream_t stream);
+int ic_moe_expert_product(const void* a, int a_stride, const void* w, long long w_expert_stride, int dtype, const int* offsets, void* out, int out_stride, int E, int N, int K, int glu, int compute_units, hipStream_t stream);
+int ic_moe_combine(const void* y, int y_stride, int dtype, const int* place, const float* weights, const void* shared, int shared_stride, int T, int top, int d, void* out, int out_stride, hipStream_t stream);
+
+// ---- stream_rows.hip: a gate on a sublayer's result, a gate on a slice of a token table -----------------------------------
+int ic_gated_norm_into_stream(const void* y, const void* g, int g_stride, int y_dtype, const float* gb, const float* w, float* x, void* copy, int copy_dtype, int T, int d, float eps, hipStream_t stream);
+int ic_token_gate(const void* z, int z_stride, const void* table, int table_stride, int dtype, const int* tokens, int col0, int n, void* out, int T, hipStream_t stream);
+
 // ---- sampling.hip -----------------------------------------------------------------------------------
 // Greedy choice per row; scratch_val / scratch_idx: 64 * n_rows elements.
 int ic_argmax(const float* logits, long long row_stride, int n_rows, int V, float* scratch_val, int* scratch_idx, int* out, hipStream_t stream);

@@ -486,3 +486,83 @@ IC_EXPORT int ic_activation(const void* in, void* out, int dtype, long long n, i
         return IC_ERR_UNSUPPORTED;
     return ic_launch_status();
 }
+
+// ---------------------------------------------------------------------------------------------
+// A sublayer's result behind a gate made from the sublayer's input:
+//   v = y[t] * sigmoid(g[t] + gb);  x[t] += v * rsqrt(mean(v^2) + eps) * w;  copy[t] = x[t] in the compute dtype.
+// g null: no gate (the kernel is then the plain norm into the stream).  One block per row.
+// ---------------------------------------------------------------------------------------------
+template <typename TY, typename TC>
+__global__ void __launch_bounds__(256)
+gated_norm_into_stream_kernel(const TY* __restrict__ y, const TY* __restrict__ g, int g_stride, const float* __restrict__ gb,
+                              const float* __restrict__ w, float* __restrict__ x, TC* __restrict__ copy, int d, float eps) {
+    __shared__ float red[16];
+    const int t = blockIdx.x;
+    const TY* yr = y + (size_t)t * d;
+    const TY* gr = g ? g + (size_t)t * g_stride : nullptr;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < d; i += blockDim.x) {
+        float v = to_f32(yr[i]);
+        if (gr) v *= 1.0f / (1.0f + expf(-(to_f32(gr[i]) + (gb ? gb[i] : 0.f))));
+        ss += v * v;
+    }
+    ss = block_sum(ss, red);
+    const float r = 1.0f / sqrtf(ss / (float)d + eps);
+    float* xr = x + (size_t)t * d;
+    for (int i = threadIdx.x; i < d; i += blockDim.x) {
+        float v = to_f32(yr[i]);
+        if (gr) v *= 1.0f / (1.0f + expf(-(to_f32(gr[i]) + (gb ? gb[i] : 0.f))));
+        const float s = xr[i] + v * r * w[i];
+        xr[i] = s;
+        if (copy) copy[(size_t)t * d + i] = from_f32<TC>(s);
+    }
+}
+
+IC_EXPORT int ic_gated_norm_into_stream(const void* y, const void* g, int g_stride, int y_dtype, const float* gb, const float* w,
+                                        float* x, void* copy, int copy_dtype, int T, int d, float eps, hipStream_t stream) {
+    if (T <= 0) return IC_OK;
+    if (d <= 0) return IC_ERR_ARG;
+    dim3 grid(T), block(256);
+    if (y_dtype == IC_F32 && (copy == nullptr || copy_dtype == IC_F32))
+        hipLaunchKernelGGL((gated_norm_into_stream_kernel<float, float>), grid, block, 0, stream, (const float*)y, (const float*)g,
+                           g_stride, gb, w, x, (float*)copy, d, eps);
+    else if (y_dtype == IC_BF16 && (copy == nullptr || copy_dtype == IC_BF16))
+        hipLaunchKernelGGL((gated_norm_into_stream_kernel<bf16, bf16>), grid, block, 0, stream, (const bf16*)y, (const bf16*)g,
+                           g_stride, gb, w, x, (bf16*)copy, d, eps);
+    else
+        return IC_ERR_UNSUPPORTED;
+    return ic_launch_status();
+}
+
+// ---------------------------------------------------------------------------------------------
+// out[t, j] = gelu_tanh(z[t, j]) * table[tokens[t], col0 + j], j < n: a gate made from the stream on a slice of the
+// token's row of a second embedding table.  gelu_tanh(z) = 0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3))).
+// ---------------------------------------------------------------------------------------------
+template <typename T>
+__global__ void __launch_bounds__(256)
+token_gate_kernel(const T* __restrict__ z, int z_stride, const T* __restrict__ table, int table_stride, const int* __restrict__ tokens,
+                  int col0, int n, T* __restrict__ out, long long total) {
+    const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= total) return;
+    const int t = (int)(i / n), j = (int)(i - (long long)t * n);
+    const float v = to_f32(z[(size_t)t * z_stride + j]);
+    const float ge = 0.5f * v * (1.0f + tanhf(0.7978845608028654f * (v + 0.044715f * v * v * v)));
+    out[i] = from_f32<T>(ge * to_f32(table[(size_t)tokens[t] * table_stride + col0 + j]));
+}
+
+IC_EXPORT int ic_token_gate(const void* z, int z_stride, const void* table, int table_stride, int dtype, const int* tokens,
+                            int col0, int n, void* out, int T, hipStream_t stream) {
+    if (T <= 0) return IC_OK;
+    if (n <= 0 || col0 < 0 || col0 + n > table_stride) return IC_ERR_ARG;
+    const long long total = (long long)T * n;
+    dim3 grid((unsigned)((total + 255) / 256)), block(256);
+    if (dtype == IC_F32)
+        hipLaunchKernelGGL(token_gate_kernel<float>, grid, block, 0, stream, (const float*)z, z_stride, (const float*)table,
+                           table_stride, tokens, col0, n, (float*)out, total);
+    else if (dtype == IC_BF16)
+        hipLaunchKernelGGL(token_gate_kernel<bf16>, grid, block, 0, stream, (const bf16*)z, z_stride, (const bf16*)table,
+                           table_stride, tokens, col0, n, (bf16*)out, total);
+    else
+        return IC_ERR_UNSUPPORTED;
+    return ic_launch_status();
+}

@@ -72,6 +72,7 @@ class LayerCacheView:
     state: Optional[torch.Tensor] = None         # [max_requests, ...] fixed-size state of this slot
     writes: bool = True
     planes: tuple = ()                           # every plane of the slot, in order (k and v are the first two)
+    blocks: Optional["LayerCacheView"] = None    # the rows kept per block of tokens (planes, block_tables), if the mixer asked for them
 
     @classmethod
     def of_planes(cls, planes, slots, block_tables, state=None) -> "LayerCacheView":
@@ -121,5 +122,5 @@ class StepContext:
     def cache_view(self, entry) -> LayerCacheView:
         v = self._views[entry.cache]
         if v.writes != entry.writes_cache:
-            v = LayerCacheView(v.k, v.v, v.slots, v.block_tables, v.state, entry.writes_cache, v.planes)
+            v = LayerCacheView(v.k, v.v, v.slots, v.block_tables, v.state, entry.writes_cache, v.planes, v.blocks)
         return v

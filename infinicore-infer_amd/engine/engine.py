@@ -101,6 +101,16 @@ class Engine:
         self.groups: List[GroupSpec] = [
             GroupSpec("window" if w else "full", nkv, dh, w, tuple(slots), planes, dims, keep)
             for (planes, nkv, dh, w, dims, keep), slots in keyed.items()]
+        # a mixer that keeps one row per block of tokens beside its tokens' rows gets a strided group for them
+        strided: Dict[tuple, List[int]] = {}
+        for slot, need in enumerate(needs):
+            if need.paged and need.block_rows:
+                strided.setdefault((need.planes, need.n_kv_heads, need.head_dim, tuple(need.plane_dims), need.block_rows), []).append(slot)
+        self._slot_strided_group = {}
+        for (planes, nkv, dh, dims, every), slots in strided.items():
+            for s in slots:
+                self._slot_strided_group[s] = len(self.groups)
+            self.groups.append(GroupSpec("full", nkv, dh, None, tuple(slots), planes, dims, 0, every))
         # positions a request may reach: the model's limit and that of every part (a table's length)
         limits = [model.spec.max_positions] + [p.position_limit() for p in model.all_parts()]
         self.max_positions = min(int(l) for l in limits if l is not None)
@@ -114,7 +124,8 @@ class Engine:
         emb_need = model.embedding_cache_need() if hasattr(model, "embedding_cache_need") else None
         if emb_need is not None and emb_need.has_state:      # what the embedding keeps per request lives with the mixers' states
             self.storage.add_state("embedding", self.max_requests, emb_need.state_shape, emb_need.state_dtype)
-        self._slot_group = {s: g for g, spec in enumerate(self.groups) for s in spec.slots}
+        self._slot_group = {s: g for g, spec in enumerate(self.groups) if spec.stride == 1 for s in spec.slots}
+        self._group_stride = [spec.stride for spec in self.groups]
         self.has_state = bool(self.storage.state)      # some mixer keeps fixed-size state per request
         self._has_window = any(g.kind == "window" for g in self.groups)
 
@@ -260,7 +271,7 @@ class Engine:
             if self.cache.has_request(e.req_id):
                 per = self.cache.pages_needed(e.req_id, len(e.tokens))
             else:
-                per = [(len(e.tokens) + self.page_size - 1) // self.page_size] * len(self.groups)
+                per = self.cache.pages_for_tokens(len(e.tokens))
             need = [a + b for a, b in zip(need, per)]
         for g, n in enumerate(need):
             if n > self.cache.free_pages(g):
@@ -362,8 +373,8 @@ class Engine:
             if req is None or not (0 <= toks[0] < vocab) or req.length >= limit:
                 return None
             found.append(req)
-            pages = req.length // ps + 1                  # pages that hold length + 1 tokens
             for g, table in enumerate(req.tables):
+                pages = self._pages_after_one(req.length, g)         # pages that hold length + 1 tokens
                 if len(table) < pages:
                     need[g] += pages - len(table)
         if len({id(r) for r in found}) != len(found):
@@ -373,13 +384,20 @@ class Engine:
                 return None
         starts = []
         for req in found:
-            pages = req.length // ps + 1
             for g, table in enumerate(req.tables):
+                pages = self._pages_after_one(req.length, g)
                 while len(table) < pages:
                     table.append(pools[g].alloc())
             starts.append(req.length)
             req.length += 1
         return starts
+
+    def _pages_after_one(self, length: int, group: int) -> int:
+        """Pages of a group that hold a request of ``length`` tokens after one more."""
+        stride = self._group_stride[group]
+        if stride == 1:
+            return length // self.page_size + 1
+        return ((length + 1) // stride + self.page_size - 1) // self.page_size
 
     def _eager_step(self, entries, starts):
         """A step that is not a replay: native code lays the batch out and launches it when the model
@@ -471,7 +489,10 @@ class Engine:
             for g in range(n_groups):
                 table = np.asarray(tables[g][r], dtype=np.int32)
                 o = offsets["slots%d" % g][0] + row0
-                a[o:o + n] = table[pos // ps] * ps + pos % ps
+                if self._group_stride[g] == 1:
+                    a[o:o + n] = table[pos // ps] * ps + pos % ps
+                else:
+                    a[o:o + n] = 0              # rows per block of tokens are addressed through the block table
                 o = offsets["tables%d" % g][0] + r * group_maxb[g]
                 a[o:o + len(table)] = np.maximum(table, 0)     # pages given back are never read; keep the index valid
                 a[o + len(table):o + group_maxb[g]] = 0
@@ -516,6 +537,9 @@ class Engine:
             if slot in self._slot_group:
                 slots, tables_g = group_views[self._slot_group[slot]]
                 ctx._views[slot] = LayerCacheView.of_planes(self.storage.planes(slot), slots, tables_g, state)
+                if slot in self._slot_strided_group:
+                    _, block_tables = group_views[self._slot_strided_group[slot]]
+                    ctx._views[slot].blocks = LayerCacheView.of_planes(self.storage.strided_planes(slot), None, block_tables)
             else:
                 ctx._views[slot] = LayerCacheView(state=state)
         return ctx
@@ -749,6 +773,10 @@ class _DecodeGraph:
                 g = engine._slot_group[slot]
                 ctx._views[slot] = LayerCacheView.of_planes(engine.storage.planes(slot), view("slots%d" % g),
                                                             view("tables%d" % g).view(R, self.maxb), state)
+                if slot in engine._slot_strided_group:
+                    sg = engine._slot_strided_group[slot]
+                    ctx._views[slot].blocks = LayerCacheView.of_planes(engine.storage.strided_planes(slot), None,
+                                                                       view("tables%d" % sg).view(R, self.maxb))
             else:
                 ctx._views[slot] = LayerCacheView(state=state)
         self.ctx = ctx
@@ -768,7 +796,8 @@ class _DecodeGraph:
             slots.append(req.state_slot)
             for g in range(len(engine.groups)):
                 table = req.tables[g]
-                a[o["slots%d" % g] + r] = table[p0 // ps] * ps + p0 % ps
+                if engine._group_stride[g] == 1:
+                    a[o["slots%d" % g] + r] = table[p0 // ps] * ps + p0 % ps
                 key = (req.serial, len(table), req.first_live[g])
                 if self._row_keys[g][r] != key:
                     base = o["tables%d" % g] + r * self.maxb

@@ -175,8 +175,7 @@ class Scheduler:
         return best, min(best_n, len(feed) - 1)
 
     def _pages_for_new(self, n_tokens: int) -> List[int]:
-        ps = self.cache.page_size
-        return [(n_tokens + ps - 1) // ps] * len(self.cache.groups)
+        return self.cache.pages_for_tokens(n_tokens)
 
     def _fits(self, need: List[int], reserved: List[int]) -> bool:
         return all(n + r <= self.cache.free_pages(g) for g, (n, r) in enumerate(zip(need, reserved)))
@@ -195,11 +194,12 @@ class Scheduler:
         decoding = [r for r in self.running if r.decoding]
         if decoding and len(decoding) <= budget:
             ps, reqs = self.cache.page_size, self.cache.requests
+            strides = [g.stride for g in self.cache.groups]
             need = [0] * ngroups
             for r in decoding:
                 e = reqs[r.task.id]
-                pages = e.length // ps + 1
                 for g, table in enumerate(e.tables):
+                    pages = e.length // ps + 1 if strides[g] == 1 else self.cache._pages_for(e.length + 1, g)
                     if len(table) < pages:
                         need[g] += pages - len(table)
             if self._fits(need, reserved):
@@ -261,9 +261,8 @@ class Scheduler:
                 if self.cache.slots.n_free == 0 and not self._evict_idle():
                     break
             n = min(self.chunk_size, len(r.feed) - shared, budget)
-            ps = self.cache.page_size
-            have = (shared + ps - 1) // ps                       # pages the kept prefix brings along
-            need = [max(0, (shared + n + ps - 1) // ps - have)] * len(self.cache.groups)
+            # pages beyond those the kept prefix brings along
+            need = [max(0, a - b) for a, b in zip(self.cache.pages_for_tokens(shared + n), self.cache.pages_for_tokens(shared))]
             while not self._fits(need, reserved) and self._evict_idle(keep=kept):
                 pass
             if not self._fits(need, reserved):

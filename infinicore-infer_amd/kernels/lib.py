@@ -133,6 +133,16 @@ _SIGNATURES = {
     "ic_attn_latent_on_matrix_cores": [_I, _I, _I],
     "ic_latent_gather": [_P, _I, _P, _I, _I, _I, _I, _I, _P, _P, _P],
     "ic_latent_softmax": [_P, _I, _P, _I, _I, _I, _I, _I, _I, _F, _P],
+    "ic_rope_pairs_store": [_P, _I, _I, _P, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P],
+    "ic_pool_blocks": [_P, _P, _P, _P, _I, _P, _I, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _P],
+    "ic_attn_pooled_generic": [_P, _I, _P, _I, _I, _P, _P, _P, _P, _P, _I, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _I, _P],
+    "ic_moe_route": [_P, _I, _I, _I, _I, _I, _I, _P, _P, _P],
+    "ic_moe_sort": [_P, _I, _I, _P, _P, _P, _P],
+    "ic_moe_gather": [_P, _I, _I, _P, _P, _I, _I, _I, _P, _P],
+    "ic_moe_expert_product": [_P, _I, _P, _LL, _I, _P, _P, _I, _I, _I, _I, _I, _I, _P],
+    "ic_moe_combine": [_P, _I, _I, _P, _P, _P, _I, _I, _I, _I, _P, _I, _P],
+    "ic_gated_norm_into_stream": [_P, _P, _I, _I, _P, _P, _P, _P, _I, _I, _I, _F, _P],
+    "ic_token_gate": [_P, _I, _P, _I, _I, _P, _I, _I, _P, _I, _P],
     "ic_sample": [_P, _LL, _I, _I, _P, _P, _P, _P, _P, _P],
     "ic_argmax": [_P, _LL, _I, _I, _P, _P, _P, _P],
     "ic_argmax_static_max_rows": [],

@@ -1173,3 +1173,188 @@ def latent_softmax(scores, probs, heads: int, first_limit: int, scale: float):
     check(get_lib().ic_latent_softmax(scores.data_ptr(), scores.stride(0), probs.data_ptr(), probs.stride(0), dtype_code(probs.dtype),
                                       M, heads, n_cols, int(first_limit), float(scale), _stream()), "latent_softmax")
     return probs
+
+
+# ---- attention over a window of tokens plus the means of the blocks before it (csrc/attn_pooled.hip) -----------------------
+def rope_pairs_store(rows, positions, freq, rot_dims: int, q_out, kcache, vcache, slots, n_heads: int, n_kv_heads: int,
+                     key_dim: int, value_dim: int, page_size: int):
+    """rows [T, >= q | k | v]: adjacent pairs of the first ``rot_dims`` entries of every query and key head turn by
+    position * f_i (``freq`` float32 [2, rot_dims / 2]: f_i rounded, and what the rounding left); q -> ``q_out``
+    [T, heads * key_dim], k and v -> the cache planes at ``slots`` (None: queries only)."""
+    _dev(rows, positions, freq, q_out, kcache, vcache, slots)
+    T = rows.shape[0]
+    nq, nk, nv = n_heads * key_dim, n_kv_heads * key_dim, n_kv_heads * value_dim
+    _need(rows.dim() == 2 and rows.stride(1) == 1 and rows.shape[1] >= nq + nk + nv, "rope_pairs_store: rows too short")
+    _need(tuple(q_out.shape) == (T, nq) and q_out.is_contiguous() and q_out.dtype == rows.dtype, "rope_pairs_store: q_out layout")
+    _need(0 <= rot_dims <= key_dim and rot_dims % 2 == 0, "rope_pairs_store: rot_dims must be even and at most the key size")
+    if rot_dims:
+        _need(freq is not None and freq.dtype == torch.float32 and freq.is_contiguous() and tuple(freq.shape) == (2, rot_dims // 2),
+              "rope_pairs_store: freq must be float32 [2, rot_dims / 2]")
+    _i32(positions, "positions")
+    _need(positions.numel() == T, "rope_pairs_store: positions/rows mismatch")
+    if slots is not None:
+        _i32(slots, "slots")
+        _need(slots.numel() == T, "rope_pairs_store: slots/rows mismatch")
+        _need(kcache.dtype == rows.dtype and vcache.dtype == rows.dtype and kcache.is_contiguous() and vcache.is_contiguous()
+              and tuple(kcache.shape[1:]) == (n_kv_heads, page_size, key_dim)
+              and tuple(vcache.shape[1:]) == (n_kv_heads, page_size, value_dim) and kcache.shape[0] == vcache.shape[0],
+              "rope_pairs_store: cache must be K [pages, kv_heads, page_size, key_dim], V [.., value_dim]")
+    check(get_lib().ic_rope_pairs_store(rows.data_ptr(), rows.stride(0), dtype_code(rows.dtype), positions.data_ptr(), _ptr(freq),
+                                        int(rot_dims), q_out.data_ptr(), _ptr(kcache) if slots is not None else None,
+                                        _ptr(vcache) if slots is not None else None, _ptr(slots), T, n_heads, n_kv_heads,
+                                        key_dim, value_dim, page_size, _stream()), "rope_pairs_store")
+    return q_out
+
+
+def _pooled_planes(kcache, vcache, kpool, vpool, n_kv_heads, key_dim, value_dim, page_size, what):
+    for k, v in ((kcache, vcache), (kpool, vpool)):
+        if k is None and v is None:
+            continue
+        _need(k is not None and v is not None and k.dtype == kcache.dtype and v.dtype == kcache.dtype and k.is_contiguous()
+              and v.is_contiguous() and tuple(k.shape[1:]) == (n_kv_heads, page_size, key_dim)
+              and tuple(v.shape[1:]) == (n_kv_heads, page_size, value_dim) and k.shape[0] == v.shape[0], what + ": cache planes")
+
+
+def pool_blocks(kcache, vcache, kpool, vpool, block_tables, pool_tables, token_req, positions, block: int, n_kv_heads: int,
+                key_dim: int, value_dim: int, page_size: int):
+    """For every token of the step that ends a block of ``block`` tokens (position p with (p + 1) % block == 0): the means of
+    the block's keys and values, read from the token cache, into row (p + 1) / block - 1 of the request's block-mean cache."""
+    _dev(kcache, vcache, kpool, vpool, block_tables, pool_tables, token_req, positions)
+    _pooled_planes(kcache, vcache, kpool, vpool, n_kv_heads, key_dim, value_dim, page_size, "pool_blocks")
+    for t, n in ((block_tables, "block_tables"), (pool_tables, "pool_tables"), (token_req, "token_req"), (positions, "positions")):
+        _need(t.dtype == torch.int32 and t.stride(-1) == 1, "pool_blocks: %s must be int32" % n)
+    T = positions.numel()
+    _need(block > 0 and token_req.numel() >= T and block_tables.dim() == 2 and pool_tables.dim() == 2, "pool_blocks: lists")
+    check(get_lib().ic_pool_blocks(kcache.data_ptr(), vcache.data_ptr(), kpool.data_ptr(), vpool.data_ptr(), dtype_code(kcache.dtype),
+                                   block_tables.data_ptr(), block_tables.stride(0), pool_tables.data_ptr(), pool_tables.stride(0),
+                                   token_req.data_ptr(), positions.data_ptr(), T, int(block), n_kv_heads, key_dim, value_dim,
+                                   page_size, _stream()), "pool_blocks")
+
+
+def attention_pooled_generic(q, out, kcache, vcache, kpool, vpool, block_tables, pool_tables, token_req, positions, bias,
+                             n_heads: int, n_kv_heads: int, key_dim: int, value_dim: int, page_size: int, scale: float,
+                             window: int, block: int):
+    """out[t, h] = sum over what position p sees of sigmoid(scale q.k + bias[h]) v: tokens j with 0 <= p - j < window
+    and blocks b with (b + 1) * block <= p - window + 1 (window 0: every earlier token, no blocks).  Any sizes up to 512."""
+    _dev(q, out, kcache, vcache, kpool, vpool, block_tables, pool_tables, token_req, positions, bias)
+    T = q.shape[0]
+    _need(q.dim() == 2 and q.stride(1) == 1 and q.shape[1] == n_heads * key_dim and out.dtype == q.dtype and out.stride(1) == 1
+          and tuple(out.shape) == (T, n_heads * value_dim) and kcache.dtype == q.dtype, "attention_pooled: q/out layout")
+    _pooled_planes(kcache, vcache, kpool, vpool, n_kv_heads, key_dim, value_dim, page_size, "attention_pooled")
+    _need(block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.stride(1) == 1, "attention_pooled: block tables")
+    pooled = bool(window and block)
+    if pooled:
+        _need(pool_tables is not None and kpool is not None and pool_tables.dtype == torch.int32 and pool_tables.dim() == 2
+              and pool_tables.stride(1) == 1, "attention_pooled: the block means' planes and tables are missing")
+    _i32(token_req, "token_req")
+    _i32(positions, "positions")
+    _need(bias is None or (bias.dtype == torch.float32 and bias.numel() == n_heads and bias.is_contiguous()), "attention_pooled: bias")
+    check(get_lib().ic_attn_pooled_generic(q.data_ptr(), q.stride(0), out.data_ptr(), out.stride(0), dtype_code(q.dtype),
+                                           kcache.data_ptr(), vcache.data_ptr(), _ptr(kpool) if pooled else None,
+                                           _ptr(vpool) if pooled else None, block_tables.data_ptr(), block_tables.stride(0),
+                                           _ptr(pool_tables) if pooled else None, pool_tables.stride(0) if pooled else 0,
+                                           token_req.data_ptr(), positions.data_ptr(), _ptr(bias), T, n_heads, n_kv_heads, key_dim,
+                                           value_dim, page_size, float(scale), int(window or 0), int(block or 0), _stream()),
+          "attention_pooled_generic")
+    return out
+
+
+# ---- routed experts (csrc/moe.hip) ----------------------------------------------------------------------------------------
+def moe_route(logits, top: int, ids, weights, mode: str = "sigmoid", renormalize: bool = False):
+    """ids[t, k], weights[t, k]: the ``top`` experts with the largest scores of float32 ``logits`` [T, E] and their scores
+    (sigmoid of the logit, or the softmax over all experts), renormalised over the chosen ones if asked."""
+    _dev(logits, ids, weights)
+    T, E = logits.shape
+    _need(logits.dtype == torch.float32 and logits.stride(1) == 1, "moe_route: float32 logits")
+    _need(ids.dtype == torch.int32 and ids.is_contiguous() and tuple(ids.shape) == (T, top) and weights.dtype == torch.float32
+          and weights.is_contiguous() and tuple(weights.shape) == (T, top), "moe_route: outputs")
+    check(get_lib().ic_moe_route(logits.data_ptr(), logits.stride(0), T, E, int(top), {"sigmoid": 0, "softmax": 1}[mode],
+                                 1 if renormalize else 0, ids.data_ptr(), weights.data_ptr(), _stream()), "moe_route")
+
+
+def moe_sort(ids, n_experts: int, offsets, order, place):
+    """The (token, choice) pairs in expert order, stable: offsets [E + 1], order [n] (sorted place -> pair), place [n]."""
+    _dev(ids, offsets, order, place)
+    n = ids.numel()
+    for t, m in ((ids, n), (offsets, n_experts + 1), (order, n), (place, n)):
+        _need(t.dtype == torch.int32 and t.is_contiguous() and t.numel() == m, "moe_sort: int32 lists")
+    check(get_lib().ic_moe_sort(ids.data_ptr(), n, int(n_experts), offsets.data_ptr(), order.data_ptr(), place.data_ptr(), _stream()),
+          "moe_sort")
+
+
+def moe_gather(h, order, weights, top: int, out):
+    """out[s] = h[order[s] // top] * weights[order[s]] (weights None: as it is)."""
+    _dev(h, order, weights, out)
+    n, d = out.shape
+    _need(h.stride(1) == 1 and h.shape[1] == d and out.is_contiguous() and out.dtype == h.dtype and order.numel() == n,
+          "moe_gather: layout")
+    _i32(order, "order")
+    _need(weights is None or (weights.dtype == torch.float32 and weights.is_contiguous() and weights.numel() == n), "moe_gather: weights")
+    check(get_lib().ic_moe_gather(h.data_ptr(), h.stride(0), dtype_code(h.dtype), order.data_ptr(), _ptr(weights), n, int(top), d,
+                                  out.data_ptr(), _stream()), "moe_gather")
+    return out
+
+
+def moe_expert_product(a, w, offsets, out, glu: bool = False, compute_units: int = 256):
+    """out[s] = a[s] W_e^T for the sorted rows s of every expert e (``offsets`` [E + 1]); ``w`` [E, N or 2N, K].  ``glu``: w
+    holds gate rows then up rows, out = silu(gate) * up.  For few rows: every row chunk streams its expert's matrix."""
+    _dev(a, w, offsets, out)
+    E, rows, K = w.shape
+    N = rows // 2 if glu else rows
+    _need(w.is_contiguous() and a.stride(1) == 1 and a.shape[1] == K and out.stride(1) == 1 and out.shape[1] == N
+          and out.shape[0] == a.shape[0] and a.dtype == w.dtype == out.dtype and (not glu or rows % 2 == 0), "moe_expert_product: layout")
+    _i32(offsets, "offsets")
+    _need(offsets.numel() == E + 1, "moe_expert_product: offsets")
+    check(get_lib().ic_moe_expert_product(a.data_ptr(), a.stride(0), w.data_ptr(), rows * K, dtype_code(a.dtype), offsets.data_ptr(),
+                                          out.data_ptr(), out.stride(0), E, N, K, 1 if glu else 0, int(compute_units), _stream()),
+          "moe_expert_product")
+    return out
+
+
+def moe_combine(y, place, weights, shared, top: int, out):
+    """out[t] = sum_k y[place[t * top + k]] * (weights[t * top + k] or 1) + (shared[t] or 0)."""
+    _dev(y, place, weights, shared, out)
+    T, d = out.shape
+    _need(y.stride(1) == 1 and y.shape[1] == d and out.stride(1) == 1 and y.dtype == out.dtype and place.numel() == T * top
+          and y.shape[0] == T * top, "moe_combine: layout")
+    _i32(place, "place")
+    _need(shared is None or (tuple(shared.shape) == (T, d) and shared.stride(1) == 1 and shared.dtype == out.dtype), "moe_combine: shared")
+    _need(weights is None or (weights.dtype == torch.float32 and weights.is_contiguous() and weights.numel() == T * top), "moe_combine: weights")
+    check(get_lib().ic_moe_combine(y.data_ptr(), y.stride(0), dtype_code(y.dtype), place.data_ptr(), _ptr(weights), _ptr(shared),
+                                   shared.stride(0) if shared is not None else 0, T, int(top), d, out.data_ptr(), out.stride(0),
+                                   _stream()), "moe_combine")
+    return out
+
+
+# ---- a gate on a sublayer's result; a gate on a slice of a token table (csrc/stream_rows.hip) ------------------------------
+def gated_norm_into_stream(y, gate, gate_bias, weight, x, eps: float, copy=None):
+    """x += rmsnorm(y * sigmoid(gate + gate_bias)) * weight, row by row (x float32, in place; ``gate`` None: no gate);
+    ``copy`` (optional) receives the new x rounded to its dtype."""
+    _dev(y, gate, gate_bias, weight, x, copy)
+    T, d = x.shape
+    _need(x.dtype == torch.float32 and x.is_contiguous() and y.is_contiguous() and tuple(y.shape) == (T, d), "gated_norm_into_stream: layout")
+    _need(weight.dtype == torch.float32 and weight.numel() == d and weight.is_contiguous(), "gated_norm_into_stream: weight must be float32 [d]")
+    if gate is not None:
+        _need(tuple(gate.shape) == (T, d) and gate.stride(1) == 1 and gate.dtype == y.dtype, "gated_norm_into_stream: gate layout")
+    _need(gate_bias is None or (gate is not None and gate_bias.dtype == torch.float32 and gate_bias.numel() == d and gate_bias.is_contiguous()),
+          "gated_norm_into_stream: gate bias must be float32 [d]")
+    if copy is not None:
+        _need(tuple(copy.shape) == (T, d) and copy.is_contiguous() and copy.dtype == y.dtype, "gated_norm_into_stream: copy layout")
+    check(get_lib().ic_gated_norm_into_stream(y.data_ptr(), _ptr(gate), gate.stride(0) if gate is not None else 0, dtype_code(y.dtype),
+                                              _ptr(gate_bias), weight.data_ptr(), x.data_ptr(), _ptr(copy),
+                                              dtype_code(copy.dtype) if copy is not None else 0, T, d, float(eps), _stream()),
+          "gated_norm_into_stream")
+    return x
+
+
+def token_gate(z, table, tokens, col0: int, out):
+    """out[t, j] = gelu_tanh(z[t, j]) * table[tokens[t], col0 + j]."""
+    _dev(z, table, tokens, out)
+    T, n = out.shape
+    _need(tuple(z.shape) == (T, n) and z.stride(1) == 1 and out.is_contiguous() and table.dim() == 2 and table.stride(1) == 1
+          and z.dtype == table.dtype == out.dtype and 0 <= col0 and col0 + n <= table.shape[1], "token_gate: layout")
+    _i32(tokens, "tokens")
+    _need(tokens.numel() == T, "token_gate: tokens/rows mismatch")
+    check(get_lib().ic_token_gate(z.data_ptr(), z.stride(0), table.data_ptr(), table.stride(0), dtype_code(z.dtype), tokens.data_ptr(),
+                                  int(col0), n, out.data_ptr(), T, _stream()), "token_gate")
+    return out

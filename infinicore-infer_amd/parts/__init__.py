@@ -2,7 +2,7 @@
 from .base import (Block, CacheNeed, FeedForward, Mixer, Norm, Part, PositionEncoding, Runtime, build_part,
                    register_part, registered_parts)
 from . import (norm, rotary, attention, swiglu, block, embedding, span_attention, dense_ffn, pair_embedding, recurrent,
-               latent_attention)      # registers the built-in parts
+               latent_attention, pooled_attention, routed_experts)      # registers the built-in parts
 from .model import DecoderModel, build_model
 
 __all__ = ["Block", "CacheNeed", "FeedForward", "Mixer", "Norm", "Part", "PositionEncoding", "Runtime",

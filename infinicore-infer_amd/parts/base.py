@@ -39,7 +39,9 @@ class CacheNeed:
     kind 'none': nothing.
     ``plane_dims``: the width of every plane when they differ (keys of 64 and values of 32 entries per head:
     (64, 32)); empty: every plane is ``head_dim`` wide.  ``keep_first``: with a window, the first tokens of a
-    sequence that stay readable for good (their pages are never given back)."""
+    sequence that stay readable for good (their pages are never given back).  ``block_rows`` P > 0: beside the tokens'
+    rows the mixer keeps one row per plane for every complete block of P tokens, in pages and with a block table of
+    their own that are never given back (``LayerCacheView.blocks``)."""
     kind: str = "none"
     n_kv_heads: int = 0
     head_dim: int = 0
@@ -49,8 +51,11 @@ class CacheNeed:
     planes: int = 2
     plane_dims: Tuple[int, ...] = ()
     keep_first: int = 0
+    block_rows: int = 0
 
     def __post_init__(self):
+        if self.block_rows < 0 or (self.block_rows and self.kind not in ("kv", "kv+state")):
+            raise ValueError("block_rows goes with a paged cache need and is not negative")
         if self.kind not in ("none", "kv", "state", "kv+state"):
             raise ValueError("cache need of kind %r (have none, kv, state, kv+state)" % (self.kind,))
         if self.paged and (self.n_kv_heads <= 0 or self.head_dim <= 0 or self.planes <= 0):

@@ -213,3 +213,117 @@ class HyperConnectionBlock(Block):
             y = self.feed_forward.forward(h, ctx)
             pending = OwedStreamWrite(y, self.hc[2][2], self.hc[2][1])
         return pending
+
+
+@register_part("block", "sandwich_gated")
+class SandwichGatedBlock(Block):
+    """Norms on both sides of every sublayer, a gate on its result, and an optional per-layer token input:
+
+        h = norm_in(x);  y = f(h) * sigmoid(R h + b);  x += norm_out(y)            (f the mixer, then the feed-forward)
+        g = gelu_tanh(G x) * S[token][c0 : c0 + dim];  x += side_norm(P g)          (after the last sublayer)
+
+    ``mixer_out_norm`` / ``feed_forward_out_norm``: the specs of the norms on the results (a layer scale rides in their
+    weight).  ``gated``: the tensors ``rg1`` [d, d], ``rg1.b`` [d] (``rg2``.. for the feed-forward); the gate is made from
+    the sublayer's input h and applied before the result's norm.  ``side``: None or {table, table_width, vocab_size,
+    first_column, dim, norm}: the tensors ``side.gate`` [dim, d], ``side.proj`` [d, dim] and a table shared by the layers,
+    of which this layer reads ``dim`` columns from ``first_column``; the gate is made from the stream itself.
+
+    The gate, the result's norm, the layer scale and the add into the float32 stream are one row kernel
+    (``ops.gated_norm_into_stream``), which also writes the stream's copy in the compute dtype when the token input wants it."""
+    graph_safe = True
+
+    def __init__(self, name, runtime, mixer=None, mixer_norm=None, feed_forward=None, feed_forward_norm=None,
+                 hidden_size: int = 0, mixer_out_norm=None, feed_forward_out_norm=None, gated: bool = True, side=None):
+        super().__init__(name, runtime, mixer, mixer_norm, feed_forward, feed_forward_norm)
+        from .base import build_part
+        if mixer is None or mixer_norm is None or mixer_out_norm is None:
+            raise ValueError("block %s: a sandwich block needs a mixer and the norms before and after it" % name)
+        if not ((feed_forward is None) == (feed_forward_norm is None) == (feed_forward_out_norm is None)):
+            raise ValueError("block %s: a feed-forward and its two norms come together, or none of them" % name)
+        self.hidden_size = int(hidden_size)
+        if self.hidden_size <= 0:
+            raise ValueError("block %s: hidden_size must be positive" % name)
+        self.mixer_out_norm = build_part("norm", mixer_out_norm, runtime)
+        self.feed_forward_out_norm = None if feed_forward_out_norm is None else build_part("norm", feed_forward_out_norm, runtime)
+        for n in (self.mixer_out_norm, self.feed_forward_out_norm):
+            if n is not None and n.deferred() is None:
+                raise ValueError("block %s: norm part %s is not a weighted RMS norm" % (name, type(n).__name__))
+        self.gated = bool(gated)
+        self.side = dict(side) if side else None
+        self.side_norm = build_part("norm", self.side["norm"], runtime) if self.side else None
+        if self.side_norm is not None and not hasattr(self.side_norm, "forward_into_stream"):
+            raise ValueError("block %s: norm part %s cannot normalise into the stream" % (name, type(self.side_norm).__name__))
+        self.gates = {}
+        self.side_gate = self.side_proj = self.side_table = None
+
+    def sub_parts(self):
+        extra = (self.mixer_out_norm, self.feed_forward_out_norm, self.side_norm)
+        return super().sub_parts() + tuple(p for p in extra if p is not None)
+
+    def _subs(self):
+        return (1, 2) if self.feed_forward is not None else (1,)
+
+    def weight_specs(self):
+        d, specs = self.hidden_size, {}
+        if self.gated:
+            for q in self._subs():
+                specs["%srg%d" % (self.name, q)] = WeightSpec((d, d))
+                specs["%srg%d.b" % (self.name, q)] = WeightSpec((d,), "vector", mean=0.0)
+        if self.side:
+            s = self.side
+            specs[s["table"]] = WeightSpec((s["vocab_size"], s["table_width"]))
+            specs[self.name + "side.gate"] = WeightSpec((s["dim"], d))
+            specs[self.name + "side.proj"] = WeightSpec((d, s["dim"]))
+        return specs
+
+    def load_weights(self, tensors):
+        if self.gated:
+            for q in self._subs():
+                self.gates[q] = (tensors["%srg%d" % (self.name, q)],
+                                 tensors["%srg%d.b" % (self.name, q)].to(torch.float32).contiguous())
+        if self.side:
+            self.side_table = tensors[self.side["table"]]
+            self.side_gate, self.side_proj = tensors[self.name + "side.gate"], tensors[self.name + "side.proj"]
+
+    def _sublayer(self, q, x, ctx, f, norm_in, norm_out, copy):
+        from .linear import linear
+        rt = self.runtime
+        h = ctx.ws.buffer("normed", tuple(x.shape), rt.dtype)
+        norm_in.forward(x, h)
+        y = f(h)
+        gate = bias = None
+        if self.gated:
+            w, bias = self.gates[q]
+            gate = ctx.ws.buffer("result_gate", tuple(x.shape), rt.dtype)
+            linear(h, w, gate, rt.gemm_impl, ws=ctx.ws)
+        weight, eps = norm_out.deferred()
+        ops.gated_norm_into_stream(y, gate, bias, weight, x, eps, copy=copy)
+
+    def forward(self, x, pending, ctx, cache):
+        from .linear import linear
+        rt = self.runtime
+        if isinstance(pending, StreamCopy):
+            pending = None
+        if pending is not None:
+            ops.residual_add(x, pending[0], pending[1])
+        # the token input reads the stream in the compute dtype: the last sublayer's kernel writes that copy along
+        copy = None
+        if self.side is not None:
+            copy = x if rt.dtype == x.dtype else ctx.ws.buffer("stream_copy", tuple(x.shape), rt.dtype)
+        has_ffn = self.feed_forward is not None
+        last_copy = None if copy is x else copy
+        self._sublayer(1, x, ctx, lambda h: self.mixer.forward(h, ctx, cache), self.mixer_norm, self.mixer_out_norm,
+                       None if has_ffn else last_copy)
+        if has_ffn:
+            self._sublayer(2, x, ctx, lambda h: self.feed_forward.forward(h, ctx), self.feed_forward_norm,
+                           self.feed_forward_out_norm, last_copy)
+        if self.side is not None:
+            s, T = self.side, x.shape[0]
+            z = ctx.ws.buffer("side_z", (T, s["dim"]), rt.dtype)
+            linear(copy, self.side_gate, z, rt.gemm_impl, ws=ctx.ws)
+            g = ctx.ws.buffer("side_g", (T, s["dim"]), rt.dtype)
+            ops.token_gate(z, self.side_table, ctx.tokens, s["first_column"], g)
+            y = ctx.ws.buffer("side_y", tuple(x.shape), rt.dtype)
+            linear(g, self.side_proj, y, rt.gemm_impl, ws=ctx.ws)
+            self.side_norm.forward_into_stream(y, x)
+        return None

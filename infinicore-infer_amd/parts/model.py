@@ -148,9 +148,23 @@ class DecoderModel:
         else:
             self.embedding.forward(ctx.tokens, x)
             pending = None
+        embedded = None
+        if any(e.adds_embedding for e in self.schedule):
+            # the embedding's output is wanted again later: a pass after the first starts from the stream plus it
+            embedded = ctx.ws.buffer("embedded", shape, torch.float32)
+            embedded.copy_(x)
         last = len(self.schedule) - 1
         for i, e in enumerate(self.schedule):
             block = self.layers[e.layer]
+            if e.adds_embedding:
+                if hasattr(pending, "settle"):
+                    pending = pending.settle(x, ctx)
+                if isinstance(pending, DeferredRows):
+                    raise RuntimeError("the embedding's output cannot join a stream whose rows are half normed")
+                if pending is not None and not isinstance(pending, StreamCopy):
+                    ops.residual_add(x, pending[0], pending[1])
+                pending = None
+                ops.residual_add(x, embedded, 1.0)
             if hasattr(pending, "settle") and not getattr(block, "accepts_owed_update", False):
                 pending = pending.settle(x, ctx)                      # an update only its own kind of block can fuse
             if isinstance(pending, StreamCopy) and not getattr(block, "accepts_stream_copy", False):
@@ -164,7 +178,9 @@ class DecoderModel:
                 continue
             # the norm that runs next, if whoever applies it can take its rows half done
             if i < last:
-                successor = self.layers[self.schedule[i + 1].layer].entry_norm()
+                # (an entry that first adds the embedding's output wants the stream itself, not half-normed rows)
+                nxt = self.schedule[i + 1]
+                successor = None if nxt.adds_embedding else self.layers[nxt.layer].entry_norm()
             elif ctx.want_rows_identity and getattr(self.head, "accepts_deferred", False):
                 successor = self.head.deferred_norm(self.final_norm)
             else:
