@@ -12,9 +12,9 @@ seeded uniform-random token ids.  One JSON line is printed.
   --workload mixed   the 1B shape's workload: 64 requests, prompts of 128..2,048 tokens, portions of 512
   --workload long    the 8B shape's workload: 4 prompts of 16,384 tokens, then decoding
   --direct           decode by calling the step function directly, without the scheduler
-  --workload designs the Fopezen, Mezinex and Daborax decoders beside the MiniCPM decoder at equal layer sizes (a few layers of three real
-                     models' sizes): prefill and decode throughput of both, with the fraction of the memory or
-                     matrix-core peak each reaches (--only fopezen|minicpm|mezinex: one of them, for a profiler)
+  --workload designs the Fopezen, Mezinex, Daborax and Fizelix decoders beside the MiniCPM decoder at equal layer sizes
+                     (a few layers of three real models' sizes): prefill and decode throughput of each, with the fraction
+                     of the memory or matrix-core peak it reaches (--only <design>: one of them, for a profiler)
 """
 import argparse
 import json
@@ -228,7 +228,20 @@ def _design_configs(z, layers):
         dab_layers.append(l)
     dab = dict(architecture="Daborax", vocab=z["vocab"], width=z["width"], norm=dict(eps=1e-5), embedding=dict(scale=1.0),
                residual_mult=0.5, layers=dab_layers)
-    return {"minicpm": mini, "fopezen": fop, "mezinex": mez, "daborax": dab}
+    # Fizelix at the same width: attention with the same heads, kv heads, key and value sizes and window as Fopezen's (half of
+    # every head rotated, one mean key and value per block of 64 tokens before the window, sigmoid weights), the state-space
+    # mixer of the Mezinex configuration; the feed-forwards are dense (the row's size) in the first and last layer and in
+    # between eight experts of a quarter of that size, two per token, beside a shared one of the same size; a gate on every
+    # sublayer's result and a token input of 64 columns per layer
+    fiz_att = dict(heads=z["heads"], kv_heads=z["kv"], dim=z["dim"], vdim=z["vdim"], scale=z["dim"] ** -0.5,
+                   mask=dict(size=z["window"], pool=64), rot=dict(base=250000.0, dims=z["dim"] // 2))
+    fiz_moe = dict(kind="moe", router=dict(experts=8, top=2), expert=dict(ff=z["ff"] // 4), shared=dict(ff=z["ff"] // 4))
+    fiz_kinds = [("attention", fiz_att, dict(kind="dense", ff=z["ff"])), ("mamba2", ssm, fiz_moe), ("attention", fiz_att, fiz_moe),
+                 ("mamba2", ssm, dict(kind="dense", ff=z["ff"]))]
+    fiz = dict(architecture="Fizelix", vocab=z["vocab"], width=z["width"], norm=dict(eps=1e-5), embedding=dict(scale=1.0),
+               logit_scale=1.0, token_side=dict(dim=64),
+               layers=[dict(type=fiz_kinds[i % 4][0], mixer=fiz_kinds[i % 4][1], mlp=fiz_kinds[i % 4][2]) for i in range(layers)])
+    return {"minicpm": mini, "fopezen": fop, "mezinex": mez, "daborax": dab, "fizelix": fiz}
 
 
 def _design_numbers(design, z, layers, kinds=None):
@@ -239,6 +252,8 @@ def _design_numbers(design, z, layers, kinds=None):
         return _mezinex_numbers(z, layers)
     if design == "daborax":
         return _daborax_numbers(z, layers)
+    if design == "fizelix":
+        return _fizelix_numbers(z, layers)
     if design == "minicpm":
         per_layer = (H + 2 * G) * dk * d + H * dk * d + 3 * d * ff
         kv = lambda n: 2 * layers * G * dk * eb * n
@@ -319,6 +334,47 @@ def _daborax_numbers(z, layers):
     return eb * weights, kv, flops
 
 
+def _fizelix_numbers(z, layers):
+    """As ``_design_numbers`` for the Fizelix configuration of ``_design_configs``.  The weights a decode step reads depend
+    on the batch: of a routed feed-forward's experts it reads those that some token chose, E (1 - (1 - top/E)^batch) on
+    average, so the first number is a function of the batch."""
+    cfg = _design_configs(z, layers)["fizelix"]
+    d, V, eb = z["width"], z["vocab"], _elem_bytes()
+    side = cfg["token_side"]["dim"]
+    fixed, per_tok_lin, scan, state_bytes = V * d, 0.0, 0.0, 0.0
+    routed = []        # (experts, top, weights of one expert) per routed feed-forward
+    spans = []         # (heads * (key + value size), kv heads * (key + value size), window, block) per attention layer
+    for l in cfg["layers"]:
+        m, mlp = l["mixer"], l["mlp"]
+        n = 2 * d * d + 2 * side * d                     # the two gates on the sublayers' results, the token input
+        if l["type"] == "attention":
+            H, G, dk, dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+            n += (H * dk + G * dk + G * dv) * d + d * H * dv
+            spans.append((H * (dk + dv), G * (dk + dv), m["mask"]["size"], m["mask"]["pool"]))
+        else:
+            inner, gn = m["heads"] * m["vdim"], m["groups"] * m["state"]
+            n += (2 * inner + 2 * gn + m["heads"]) * d + d * inner
+            state_bytes += 2 * 4 * (inner * m["state"] + (m["conv"] - 1) * (inner + 2 * gn))
+            scan += 6.0 * inner * m["state"]
+        active = n
+        if mlp["kind"] == "dense":
+            n += 3 * d * mlp["ff"]
+            active = n
+        else:
+            E, top, one = mlp["router"]["experts"], mlp["router"]["top"], 3 * d * mlp["expert"]["ff"]
+            n += E * d + 3 * d * mlp["shared"]["ff"]
+            active = n + top * one
+            routed.append((E, top, one))
+        fixed += n
+        per_tok_lin += 2.0 * active
+    seen = lambda n, w, p: min(n, w) + max(0, n - w) // p
+    weights = lambda batch: eb * (fixed + sum(E * (1.0 - (1.0 - top / E) ** batch) * one for E, top, one in routed))
+    kv = lambda n: sum(g * eb * seen(n, w, p) for _, g, w, p in spans) + state_bytes
+    flops = lambda T: (T * (per_tok_lin + scan) + sum(2.0 * h * sum(seen(i + 1, w, p) for i in range(T)) for h, _, w, p in spans)
+                       + 2.0 * V * d)
+    return weights, kv, flops
+
+
 def run_designs(args):
     """Prefill and decode of the two decoders at equal layer sizes.  Decoding calls the step function directly (recorded
     steps), greedy sampling on the device; a row gives tokens/s and what fraction of the memory bandwidth (decoding:
@@ -356,7 +412,7 @@ def run_designs(args):
             for b in batches:
                 dt, ctx = time_decode(engine, b, args.steps, args.warmup, z["vocab"], seed=b)
                 row["decode"]["batch %d" % b] = {"tokens_per_s": round(b / dt, 1), "ms_per_step": round(dt * 1e3, 4),
-                                                 "frac_of_hbm_peak": round((weights + b * kv(ctx)) / dt / 1e9 / HBM_PEAK_GBS, 4)}
+                                                 "frac_of_hbm_peak": round(((weights(b) if callable(weights) else weights) + b * kv(ctx)) / dt / 1e9 / HBM_PEAK_GBS, 4)}
             rows.append(row)
             print(json.dumps(row), file=sys.stderr, flush=True)
             del engine, model
@@ -454,7 +510,7 @@ def main():
     ap.add_argument("--layers", type=int, default=0, help="fewer layers than the shape has (0: all)")
     ap.add_argument("--shape", default=None, choices=sorted(SHAPES), help="2b is the benchmark's configuration (default; 1b for --workload mixed)")
     ap.add_argument("--sizes", default=None, help="--workload designs: comma-separated sizes (default: all of 2b-like, 8b-like, 1b-like)")
-    ap.add_argument("--only", default=None, choices=["fopezen", "minicpm", "mezinex", "daborax"], help="--workload designs: one design only")
+    ap.add_argument("--only", default=None, choices=["fopezen", "minicpm", "mezinex", "daborax", "fizelix"], help="--workload designs: one design only")
     ap.add_argument("--workload", default="decode", choices=["decode", "mixed", "long", "designs"],
                     help="decode: the benchmark (prefill of one prompt, decode steps at fixed batches); "
                          "mixed: 64 requests of 128..2048 prompt tokens through the scheduler, --steps tokens generated each; "

@@ -39,11 +39,12 @@ class GroupSpec:
     planes: int = 2                     # tensors per slot (keys and values: 2; one latent per token: 1)
     plane_dims: tuple = ()              # width of each plane when they differ; empty: all head_dim
     keep_first: int = 0                 # 'window': the first tokens that stay readable for good
-    stride: int = 1                     # tokens per row: a group with stride P holds one row for every COMPLETE block of P tokens
+    stride: int = 1                     # tokens per row of a group ``of_blocks``
+    of_blocks: bool = False             # the group holds one row for every COMPLETE block of ``stride`` tokens, not one per token
 
     def __post_init__(self):
-        if self.stride < 1 or (self.stride > 1 and self.kind != "full"):
-            raise CacheError("a group's stride is a positive token count, and a strided group keeps every row")
+        if self.stride < 1 or (self.stride > 1 and not self.of_blocks) or (self.of_blocks and self.kind != "full"):
+            raise CacheError("a group's stride is a positive token count, goes with of_blocks, and a group of blocks keeps every row")
         if self.kind not in ("full", "window"):
             raise CacheError("group kind must be 'full' or 'window'")
         if self.kind == "window" and not (self.window and self.window > 0):

@@ -36,7 +36,7 @@ class CacheStorage:
                                            dtype=dtype, device=device) for w in dims)
             self.group_planes.append(planes)
             for i, s in enumerate(spec.slots):
-                (self._strided_index if spec.stride > 1 else self._slot_index)[s] = (g, i)
+                (self._strided_index if spec.of_blocks else self._slot_index)[s] = (g, i)
         self.state: Dict[int, torch.Tensor] = {}               # cache slot -> [max_requests, ...]
         self._kv_views: Dict[object, tuple] = {}
         self._copy_idx = None                                  # (pinned, device) page ids of copy_pages, kept between calls

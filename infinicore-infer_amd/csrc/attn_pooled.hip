@@ -116,14 +116,13 @@ pool_blocks_kernel(const T* __restrict__ kcache, const T* __restrict__ vcache, T
     const int* bt = block_tables + (size_t)token_req[t] * bt_stride;
     const int* pt = pool_tables + (size_t)token_req[t] * pt_stride;
     const long long orow = cache_row(pt, b, page_size, nkvh, g);
-    const float inv = 1.0f / (float)P;
     for (int d = lane; d < dk + dv; d += 64) {
         const bool key = d < dk;
         const int c = key ? d : d - dk, w = key ? dk : dv;
         const T* plane = key ? kcache : vcache;
         float s = 0.f;
         for (int j = 0; j < P; ++j) s += to_f32(plane[cache_row(bt, b * P + j, page_size, nkvh, g) * w + c]);
-        (key ? kpool : vpool)[orow * w + c] = from_f32<T>(s * inv);
+        (key ? kpool : vpool)[orow * w + c] = from_f32<T>(s / (float)P);
     }
 }
 
@@ -253,5 +252,375 @@ IC_EXPORT int ic_attn_pooled_generic(const void* q, int q_stride, void* out, int
                            page_size, scale, window, P);
     else
         return IC_ERR_UNSUPPORTED;
+    return ic_launch_status();
+}
+
+// =============================================================================================
+// Single new tokens, split over what a token sees so that few requests fill the chip.
+//
+// Pass 1, grid (splits, kv heads, tokens), 256 threads: the seen items of a token are numbered 0 .. total - 1 (the
+// blocks, then the window's tokens); a block streams its share once and serves every query head of the kv head, four
+// at a time.  DK / VEC lanes share an item (VEC = 16 bytes of elements), so a wave reads whole rows; the same lanes
+// read the value row in 16-byte pieces.  The weights are not normalised, so shares simply add up: lane groups,
+// waves, and (pass 2) splits.  With one split pass 1 writes the result itself.
+// =============================================================================================
+template <typename T> struct PoolVec;
+template <> struct PoolVec<float> {
+    static constexpr int N = 4;
+    __device__ static void load(const float* p, float* o) {
+        const float4 v = *reinterpret_cast<const float4*>(p);
+        o[0] = v.x; o[1] = v.y; o[2] = v.z; o[3] = v.w;
+    }
+};
+template <> struct PoolVec<bf16> {
+    static constexpr int N = 8;
+    __device__ static void load(const bf16* p, float* o) {
+        const uint4 v = *reinterpret_cast<const uint4*>(p);
+        o[0] = __uint_as_float(v.x << 16); o[1] = __uint_as_float(v.x & 0xffff0000u);
+        o[2] = __uint_as_float(v.y << 16); o[3] = __uint_as_float(v.y & 0xffff0000u);
+        o[4] = __uint_as_float(v.z << 16); o[5] = __uint_as_float(v.z & 0xffff0000u);
+        o[6] = __uint_as_float(v.w << 16); o[7] = __uint_as_float(v.w & 0xffff0000u);
+    }
+};
+
+constexpr int kPdHeads = 4;      // query heads served per walk
+
+template <typename T, int DK, int DV>
+__global__ void __launch_bounds__(256)
+attn_pooled_decode_kernel(const T* __restrict__ q, int q_stride, const T* __restrict__ kcache, const T* __restrict__ vcache,
+                          const T* __restrict__ kpool, const T* __restrict__ vpool, const int* __restrict__ block_tables,
+                          int bt_stride, const int* __restrict__ pool_tables, int pt_stride, const int* __restrict__ tok_list,
+                          const int* __restrict__ token_req, const int* __restrict__ positions, const float* __restrict__ bias,
+                          float* __restrict__ parts, T* __restrict__ out, int out_stride, int nh, int nkvh, int page_size,
+                          float scale, int window, int P, int n_tok, int nsplit) {
+    constexpr int VEC = PoolVec<T>::N;
+    constexpr int LPK = DK / VEC;                   // lanes that share an item
+    constexpr int KPW = 64 / LPK;                   // items a wave takes at a time
+    constexpr int VP = DV / VEC;                    // 16-byte pieces of a value row
+    constexpr int NP = (VP + LPK - 1) / LPK;        // pieces a lane takes
+    static_assert(LPK <= 64 && 64 % LPK == 0 && DV % VEC == 0, "rows in whole 16-byte pieces");
+    __shared__ float qs[kPdHeads][DK];
+    __shared__ float red[4][kPdHeads][DV];
+
+    const int split = blockIdx.x, kvh = blockIdx.y, ti = blockIdx.z;
+    const int t = tok_list ? tok_list[ti] : ti;
+    const int G = nh / nkvh;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int sub = lane % LPK, grp = lane / LPK;
+    const int pos = positions[t];
+    const int* bt = block_tables + (size_t)token_req[t] * bt_stride;
+    const int* pt = pool_tables ? pool_tables + (size_t)token_req[t] * pt_stride : nullptr;
+    const PooledSpan span = pooled_span(pos, window, pt ? P : 0);
+    const int per = (span.total + nsplit - 1) / nsplit;
+    const int i0 = split * per, i1 = min(span.total, i0 + per);
+
+    for (int g0 = 0; g0 < G; g0 += kPdHeads) {
+        const int gq = min(kPdHeads, G - g0);
+        __syncthreads();
+        for (int i = tid; i < gq * DK; i += 256) {
+            const int g = i / DK, d = i - g * DK;
+            qs[g][d] = to_f32(q[(size_t)t * q_stride + (size_t)(kvh * G + g0 + g) * DK + d]);
+        }
+        __syncthreads();
+        float qr[kPdHeads][VEC], hb[kPdHeads], acc[kPdHeads][NP][VEC];
+#pragma unroll
+        for (int g = 0; g < kPdHeads; ++g) {
+            hb[g] = (bias && g < gq) ? bias[kvh * G + g0 + g] : 0.f;
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) qr[g][j] = g < gq ? qs[g][sub * VEC + j] : 0.f;
+#pragma unroll
+            for (int n = 0; n < NP; ++n)
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) acc[g][n][j] = 0.f;
+        }
+        for (int it = i0 + wave * KPW + grp; it < i1; it += 4 * KPW) {
+            const bool pooled = it < span.nb;
+            const long long rowi = pooled ? cache_row(pt, it, page_size, nkvh, kvh)
+                                          : cache_row(bt, span.lo + (it - span.nb), page_size, nkvh, kvh);
+            float kf[VEC], vf[NP][VEC];
+            PoolVec<T>::load((pooled ? kpool : kcache) + rowi * DK + sub * VEC, kf);
+#pragma unroll
+            for (int n = 0; n < NP; ++n) {
+                const int piece = sub + n * LPK;
+                if (piece < VP) PoolVec<T>::load((pooled ? vpool : vcache) + rowi * DV + piece * VEC, vf[n]);
+                else
+#pragma unroll
+                    for (int j = 0; j < VEC; ++j) vf[n][j] = 0.f;
+            }
+#pragma unroll
+            for (int g = 0; g < kPdHeads; ++g) {
+                float d = 0.f;
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) d += kf[j] * qr[g][j];
+                d = group_sum<LPK>(d);
+                const float p = sigmoid_acc(d * scale + hb[g]);
+#pragma unroll
+                for (int n = 0; n < NP; ++n)
+#pragma unroll
+                    for (int j = 0; j < VEC; ++j) acc[g][n][j] += p * vf[n][j];
+            }
+        }
+        // lanes with the same place in their group hold shares of the same columns
+#pragma unroll
+        for (int g = 0; g < kPdHeads; ++g)
+#pragma unroll
+            for (int n = 0; n < NP; ++n)
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) {
+                    float v = acc[g][n][j];
+#pragma unroll
+                    for (int o = LPK; o < 64; o <<= 1) v += __shfl_xor(v, o, kWave);
+                    acc[g][n][j] = v;
+                }
+        if (grp == 0) {
+#pragma unroll
+            for (int g = 0; g < kPdHeads; ++g)
+#pragma unroll
+                for (int n = 0; n < NP; ++n) {
+                    const int piece = sub + n * LPK;
+                    if (piece < VP)
+#pragma unroll
+                        for (int j = 0; j < VEC; ++j) red[wave][g][piece * VEC + j] = acc[g][n][j];
+                }
+        }
+        __syncthreads();
+        for (int i = tid; i < gq * DV; i += 256) {
+            const int g = i / DV, d = i - g * DV;
+            const float v = red[0][g][d] + red[1][g][d] + red[2][g][d] + red[3][g][d];
+            const int h = kvh * G + g0 + g;
+            if (nsplit == 1) out[(size_t)t * out_stride + (size_t)h * DV + d] = from_f32<T>(v);
+            else parts[(((size_t)split * n_tok + ti) * nh + h) * DV + d] = v;
+        }
+    }
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+attn_pooled_merge_kernel(const float* __restrict__ parts, const int* __restrict__ tok_list, T* __restrict__ out, int out_stride,
+                         int n_tok, int width, int nsplit) {
+    const int ti = blockIdx.x, t = tok_list ? tok_list[ti] : ti;
+    for (int i = threadIdx.x; i < width; i += blockDim.x) {
+        float v = 0.f;
+        for (int s = 0; s < nsplit; ++s) v += parts[((size_t)s * n_tok + ti) * width + i];
+        out[(size_t)t * out_stride + i] = from_f32<T>(v);
+    }
+}
+
+IC_EXPORT int ic_attn_pooled_decode_supported(int dtype, int dk, int dv) {
+    return (dtype == IC_F32 || dtype == IC_BF16) && (dk == 64 || dk == 128) && (dv == 64 || dv == 128);
+}
+
+IC_EXPORT int ic_attn_pooled_decode(const void* q, int q_stride, void* out, int out_stride, int dtype, const void* kcache,
+                                    const void* vcache, const void* kpool, const void* vpool, const int* block_tables,
+                                    int bt_stride, const int* pool_tables, int pt_stride, const int* tok_list,
+                                    const int* token_req, const int* positions, const float* bias, float* parts, int n_tok,
+                                    int nh, int nkvh, int dk, int dv, int page_size, float scale, int window, int P, int nsplit,
+                                    hipStream_t stream) {
+    if (n_tok <= 0) return IC_OK;
+    if (!ic_attn_pooled_decode_supported(dtype, dk, dv)) return IC_ERR_UNSUPPORTED;
+    if (nh <= 0 || nkvh <= 0 || nh % nkvh || page_size <= 0 || window < 0 || P < 0 || nsplit < 1 || nsplit > 64 || nkvh > 65535 ||
+        n_tok > 65535 || (nsplit > 1 && parts == nullptr))
+        return IC_ERR_ARG;
+    if (P > 0 && window > 0 && (pool_tables == nullptr || kpool == nullptr || vpool == nullptr)) return IC_ERR_ARG;
+    dim3 grid((unsigned)nsplit, (unsigned)nkvh, (unsigned)n_tok), block(256);
+#define IC_PD(TT, K, V)                                                                                                 \
+    hipLaunchKernelGGL((attn_pooled_decode_kernel<TT, K, V>), grid, block, 0, stream, (const TT*)q, q_stride,             \
+                       (const TT*)kcache, (const TT*)vcache, (const TT*)kpool, (const TT*)vpool, block_tables, bt_stride, \
+                       pool_tables, pt_stride, tok_list, token_req, positions, bias, parts, (TT*)out, out_stride, nh, nkvh, \
+                       page_size, scale, window, P, n_tok, nsplit)
+#define IC_PD_T(TT)                                                                                                     \
+    do {                                                                                                                \
+        if (dk == 64 && dv == 64) IC_PD(TT, 64, 64);                                                                    \
+        else if (dk == 64) IC_PD(TT, 64, 128);                                                                          \
+        else if (dv == 64) IC_PD(TT, 128, 64);                                                                          \
+        else IC_PD(TT, 128, 128);                                                                                       \
+    } while (0)
+    if (dtype == IC_F32) IC_PD_T(float); else IC_PD_T(bf16);
+#undef IC_PD_T
+#undef IC_PD
+    int st = ic_launch_status();
+    if (st != IC_OK || nsplit == 1) return st;
+    if (dtype == IC_F32)
+        hipLaunchKernelGGL(attn_pooled_merge_kernel<float>, dim3(n_tok), dim3(256), 0, stream, parts, tok_list, (float*)out,
+                           out_stride, n_tok, nh * dv, nsplit);
+    else
+        hipLaunchKernelGGL(attn_pooled_merge_kernel<bf16>, dim3(n_tok), dim3(256), 0, stream, parts, tok_list, (bf16*)out,
+                           out_stride, n_tok, nh * dv, nsplit);
+    return ic_launch_status();
+}
+
+// =============================================================================================
+// Prompt portions on the matrix cores (bfloat16; key and value sizes 32, 64, 128).
+//
+// Grid (query tiles * heads), tile-major, 256 threads.  A tile is up to 128 consecutive tokens of one request (int4:
+// request row, first token row, rows, first position); wave w owns rows 32w..32w+31.  What the tile may see is walked 64
+// items at a time: first the blocks' means that its last row sees, then the tokens from the first row's window to the
+// last row.  A step's keys and values pass through LDS as padded rows.  S^T = K Q^T with v_mfma_f32_32x32x16_bf16: a lane
+// holds 32 items of ONE query, so the mask and the sigmoid need no cross-lane step and the weights are already the B
+// operand of O^T = V^T P^T, whose A operand comes out of LDS through the transposing read.  Operand layout (lane l,
+// h = l/32): A[i = l%32][k = 8h..8h+7], B[k = 8h..8h+7][j = l%32], D[i = 8(r/4) + 4h + r%4][j = l%32].
+// An item outside the run a step walks is replaced by the last one inside when it is loaded, and masked.
+// =============================================================================================
+typedef __bf16 pl_bf16x8 __attribute__((ext_vector_type(8)));
+typedef float pl_v16f __attribute__((ext_vector_type(16)));
+typedef float pl_v8f __attribute__((ext_vector_type(8)));
+typedef short pl_v4s __attribute__((ext_vector_type(4)));
+typedef unsigned pl_v4u __attribute__((ext_vector_type(4)));
+
+constexpr int kPlRows = 128;
+constexpr int kPlItems = 64;
+
+template <int DK, int DV>
+__global__ void __launch_bounds__(256, 2)
+attn_pooled_prefill_kernel(const uint16_t* __restrict__ q, int q_stride, uint16_t* __restrict__ out, int out_stride,
+                           const uint16_t* __restrict__ kcache, const uint16_t* __restrict__ vcache,
+                           const uint16_t* __restrict__ kpool, const uint16_t* __restrict__ vpool,
+                           const int* __restrict__ block_tables, int bt_stride, const int* __restrict__ pool_tables, int pt_stride,
+                           const int4* __restrict__ tiles, const float* __restrict__ bias, int nh, int nkvh, int page_size,
+                           float scale, int window, int P) {
+    constexpr int NC = DK / 16, ND = DV / 32, PK = DK + 8, PV = DV + 8, KCH = DK / 8, VCH = DV / 8;
+    constexpr int NLK = kPlItems * KCH / 256, NLV = kPlItems * VCH / 256;
+    static_assert(DK % 32 == 0 && DV % 32 == 0, "a step's rows split evenly over the block");
+    __shared__ __attribute__((aligned(16))) uint16_t Ks[kPlItems * PK];
+    __shared__ __attribute__((aligned(16))) uint16_t Vs[kPlItems * PV];
+
+    const int slot = (int)blockIdx.x;
+    const int h = slot % nh;
+    const int4 tile = tiles[slot / nh];
+    const int req = tile.x, row0 = tile.y, n_rows = tile.z, pos0 = tile.w;
+    const int kvh = h / (nh / nkvh);
+    const int* bt = block_tables + (size_t)req * bt_stride;
+    const int* pt = pool_tables ? pool_tables + (size_t)req * pt_stride : nullptr;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int lq = lane & 31, half = lane >> 5;
+    const bool wave_ok = 32 * wave < n_rows;
+    const int my_row = min(32 * wave + lq, n_rows - 1);
+    const int qpos = pos0 + my_row;
+    const PooledSpan mine = pooled_span(qpos, window, pt ? P : 0);
+    const int last_pos = pos0 + n_rows - 1;
+    const int lo_min = pooled_span(pos0, window, 0).lo;
+    const int nb_max = pooled_span(last_pos, window, pt ? P : 0).nb;
+    const int block_steps = (nb_max + kPlItems - 1) / kPlItems;
+    const int n_steps = block_steps + (last_pos - lo_min + kPlItems) / kPlItems;
+    const float hb = bias ? bias[h] : 0.f;
+
+    pl_bf16x8 qf[NC];
+    {
+        const uint16_t* qp = q + (size_t)(row0 + my_row) * q_stride + (size_t)h * DK + 8 * half;
+#pragma unroll
+        for (int c = 0; c < NC; ++c) qf[c] = *reinterpret_cast<const pl_bf16x8*>(qp + 16 * c);
+    }
+    pl_v16f oacc[ND];
+#pragma unroll
+    for (int i = 0; i < ND; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) oacc[i][r] = 0.f;
+    const int vrow = 4 * half + ((lane & 15) >> 2);
+    const int vcol = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+
+    for (int s = 0; s < n_steps; ++s) {
+        const bool pooled = s < block_steps;
+        const int base = pooled ? kPlItems * s : lo_min + kPlItems * (s - block_steps);
+        const int hi = pooled ? nb_max - 1 : last_pos;
+        const uint16_t* kplane = pooled ? kpool : kcache;
+        const uint16_t* vplane = pooled ? vpool : vcache;
+        const int* table = pooled ? pt : bt;
+        __syncthreads();                                   // the step before has been read
+#pragma unroll
+        for (int i = 0; i < NLK; ++i) {
+            const int idx = tid + i * 256, kk = idx / KCH, c = idx - kk * KCH;
+            const long long rowi = cache_row(table, min(base + kk, hi), page_size, nkvh, kvh);
+            *reinterpret_cast<pl_v4u*>(Ks + kk * PK + c * 8) = *reinterpret_cast<const pl_v4u*>(kplane + rowi * DK + c * 8);
+        }
+#pragma unroll
+        for (int i = 0; i < NLV; ++i) {
+            const int idx = tid + i * 256, kk = idx / VCH, c = idx - kk * VCH;
+            const long long rowi = cache_row(table, min(base + kk, hi), page_size, nkvh, kvh);
+            *reinterpret_cast<pl_v4u*>(Vs + kk * PV + c * 8) = *reinterpret_cast<const pl_v4u*>(vplane + rowi * DV + c * 8);
+        }
+        __syncthreads();
+        if (!wave_ok) continue;
+        pl_v16f sacc[2];
+#pragma unroll
+        for (int tt = 0; tt < 2; ++tt) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) sacc[tt][r] = 0.f;
+#pragma unroll
+            for (int c = 0; c < NC; ++c) {
+                const pl_bf16x8 a = *reinterpret_cast<const pl_bf16x8*>(Ks + (32 * tt + lq) * PK + 16 * c + 8 * half);
+                sacc[tt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qf[c], sacc[tt], 0, 0, 0);
+            }
+        }
+        // weights: sigmoid(scale s + bias) where this lane's query sees the item, else nothing
+        const int lim_lo = pooled ? 0 : mine.lo, lim_hi = pooled ? mine.nb - 1 : qpos;
+#pragma unroll
+        for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int item = base + 32 * tt + 8 * (r >> 2) + 4 * half + (r & 3);
+                const float z = fmaf(sacc[tt][r], scale, hb);
+                const float p = __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(-1.4426950408889634f * z));
+                sacc[tt][r] = (item >= lim_lo && item <= lim_hi) ? p : 0.f;
+            }
+#pragma unroll
+        for (int kc = 0; kc < 4; ++kc) {
+            const int tt = kc >> 1, r0 = 8 * (kc & 1);
+            pl_v8f pf;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) pf[e] = sacc[tt][r0 + e];
+            const pl_bf16x8 b = __builtin_convertvector(pf, pl_bf16x8);
+#pragma unroll
+            for (int dt = 0; dt < ND; ++dt) {
+                const uint16_t* vp = Vs + (16 * kc + vrow) * PV + 32 * dt + vcol;
+                const pl_v4s lo4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((pl_v4s __attribute__((address_space(3)))*)vp);
+                const pl_v4s hi4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((pl_v4s __attribute__((address_space(3)))*)(vp + 8 * PV));
+                const pl_bf16x8 a = __builtin_bit_cast(pl_bf16x8, __builtin_shufflevector(lo4, hi4, 0, 1, 2, 3, 4, 5, 6, 7));
+                oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, oacc[dt], 0, 0, 0);
+            }
+        }
+    }
+    if (32 * wave + lq < n_rows) {
+        uint16_t* op = out + (size_t)(row0 + my_row) * out_stride + (size_t)h * DV;
+#pragma unroll
+        for (int dt = 0; dt < ND; ++dt)
+#pragma unroll
+            for (int r4 = 0; r4 < 4; ++r4) {
+                uint2 v;
+                v.x = (uint32_t)f32_to_bf16_bits(oacc[dt][4 * r4]) | ((uint32_t)f32_to_bf16_bits(oacc[dt][4 * r4 + 1]) << 16);
+                v.y = (uint32_t)f32_to_bf16_bits(oacc[dt][4 * r4 + 2]) | ((uint32_t)f32_to_bf16_bits(oacc[dt][4 * r4 + 3]) << 16);
+                *reinterpret_cast<uint2*>(op + 32 * dt + 8 * r4 + 4 * half) = v;
+            }
+    }
+}
+
+IC_EXPORT int ic_attn_pooled_prefill_supported(int dtype, int dk, int dv) {
+    auto ok = [](int d) { return d == 32 || d == 64 || d == 128; };
+    return dtype == IC_BF16 && ok(dk) && ok(dv);
+}
+
+IC_EXPORT int ic_attn_pooled_prefill(const void* q, int q_stride, void* out, int out_stride, int dtype, const void* kcache,
+                                     const void* vcache, const void* kpool, const void* vpool, const int* block_tables,
+                                     int bt_stride, const int* pool_tables, int pt_stride, const int* tiles, int n_tiles,
+                                     const float* bias, int nh, int nkvh, int dk, int dv, int page_size, float scale,
+                                     int window, int P, hipStream_t stream) {
+    if (n_tiles <= 0) return IC_OK;
+    if (!ic_attn_pooled_prefill_supported(dtype, dk, dv)) return IC_ERR_UNSUPPORTED;
+    if (nh <= 0 || nkvh <= 0 || nh % nkvh || page_size <= 0 || window < 0 || P < 0 || (q_stride % 8) || (out_stride % 4) ||
+        ((uintptr_t)q % 16) || ((uintptr_t)out % 8) || (long long)n_tiles * nh > 0x7fffffffLL)
+        return IC_ERR_ARG;
+    if (P > 0 && window > 0 && (pool_tables == nullptr || kpool == nullptr || vpool == nullptr)) return IC_ERR_ARG;
+    dim3 grid((unsigned)(n_tiles * nh)), block(256);
+#define IC_PP(K, V)                                                                                                     \
+    hipLaunchKernelGGL((attn_pooled_prefill_kernel<K, V>), grid, block, 0, stream, (const uint16_t*)q, q_stride,          \
+                       (uint16_t*)out, out_stride, (const uint16_t*)kcache, (const uint16_t*)vcache, (const uint16_t*)kpool, \
+                       (const uint16_t*)vpool, block_tables, bt_stride, pool_tables, pt_stride, (const int4*)tiles, bias, nh, \
+                       nkvh, page_size, scale, window, P)
+#define IC_PP_V(K)                                                                                                      \
+    do {                                                                                                                \
+        if (dv == 32) IC_PP(K, 32); else if (dv == 64) IC_PP(K, 64); else IC_PP(K, 128);                                 \
+    } while (0)
+    if (dk == 32) IC_PP_V(32); else if (dk == 64) IC_PP_V(64); else IC_PP_V(128);
+#undef IC_PP_V
+#undef IC_PP
     return ic_launch_status();
 }

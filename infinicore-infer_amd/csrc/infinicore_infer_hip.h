@@ -158,6 +158,12 @@ int ic_rope_pairs_store(const void* rows, int row_stride, int dtype, const int* 
 int ic_pool_blocks(const void* kcache, const void* vcache, void* kpool, void* vpool, int dtype, const int* block_tables, int bt_stride, const int* pool_tables, int pt_stride, const int* token_req, const int* positions, int T, int P, int nkvh, int dk, int dv, int page_size, hipStream_t stream);
 // out_i = sum over seen tokens and blocks of sigmoid(scale q.k + bias[h]) v; any sizes up to 512, float32 or bfloat16.
 int ic_attn_pooled_generic(const void* q, int q_stride, void* out, int out_stride, int dtype, const void* kcache, const void* vcache, const void* kpool, const void* vpool, const int* block_tables, int bt_stride, const int* pool_tables, int pt_stride, const int* token_req, const int* positions, const float* bias, int T, int nh, int nkvh, int dk, int dv, int page_size, float scale, int window, int P, hipStream_t stream);
+// Single tokens, split over what they see (key and value sizes 64 or 128; parts: float32 [nsplit, n_tok, nh, dv] when nsplit > 1).
+int ic_attn_pooled_decode_supported(int dtype, int dk, int dv);
+int ic_attn_pooled_decode(const void* q, int q_stride, void* out, int out_stride, int dtype, const void* kcache, const void* vcache, const void* kpool, const void* vpool, const int* block_tables, int bt_stride, const int* pool_tables, int pt_stride, const int* tok_list, const int* token_req, const int* positions, const float* bias, float* parts, int n_tok, int nh, int nkvh, int dk, int dv, int page_size, float scale, int window, int P, int nsplit, hipStream_t stream);
+// Prompt portions on the matrix cores (bfloat16; key and value sizes 32, 64, 128).  tiles as for ic_attn_prefill, rows <= 128.
+int ic_attn_pooled_prefill_supported(int dtype, int dk, int dv);
+int ic_attn_pooled_prefill(const void* q, int q_stride, void* out, int out_stride, int dtype, const void* kcache, const void* vcache, const void* kpool, const void* vpool, const int* block_tables, int bt_stride, const int* pool_tables, int pt_stride, const int* tiles, int n_tiles, const float* bias, int nh, int nkvh, int dk, int dv, int page_size, float scale, int window, int P, hipStream_t stream);
 
 // ---- moe.hip: routed experts --------------------------------------------------------------------------------------
 int ic_moe_route(const float* z, int z_stride, int T, int E, int top, int mode, int renorm, int* ids, float* weights, hipStream_t stream);

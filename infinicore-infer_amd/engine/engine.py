@@ -110,7 +110,7 @@ class Engine:
         for (planes, nkv, dh, dims, every), slots in strided.items():
             for s in slots:
                 self._slot_strided_group[s] = len(self.groups)
-            self.groups.append(GroupSpec("full", nkv, dh, None, tuple(slots), planes, dims, 0, every))
+            self.groups.append(GroupSpec("full", nkv, dh, None, tuple(slots), planes, dims, 0, every, True))
         # positions a request may reach: the model's limit and that of every part (a table's length)
         limits = [model.spec.max_positions] + [p.position_limit() for p in model.all_parts()]
         self.max_positions = min(int(l) for l in limits if l is not None)
@@ -124,8 +124,9 @@ class Engine:
         emb_need = model.embedding_cache_need() if hasattr(model, "embedding_cache_need") else None
         if emb_need is not None and emb_need.has_state:      # what the embedding keeps per request lives with the mixers' states
             self.storage.add_state("embedding", self.max_requests, emb_need.state_shape, emb_need.state_dtype)
-        self._slot_group = {s: g for g, spec in enumerate(self.groups) if spec.stride == 1 for s in spec.slots}
+        self._slot_group = {s: g for g, spec in enumerate(self.groups) if not spec.of_blocks for s in spec.slots}
         self._group_stride = [spec.stride for spec in self.groups]
+        self._group_of_blocks = [spec.of_blocks for spec in self.groups]
         self.has_state = bool(self.storage.state)      # some mixer keeps fixed-size state per request
         self._has_window = any(g.kind == "window" for g in self.groups)
 
@@ -394,10 +395,9 @@ class Engine:
 
     def _pages_after_one(self, length: int, group: int) -> int:
         """Pages of a group that hold a request of ``length`` tokens after one more."""
-        stride = self._group_stride[group]
-        if stride == 1:
+        if not self._group_of_blocks[group]:
             return length // self.page_size + 1
-        return ((length + 1) // stride + self.page_size - 1) // self.page_size
+        return ((length + 1) // self._group_stride[group] + self.page_size - 1) // self.page_size
 
     def _eager_step(self, entries, starts):
         """A step that is not a replay: native code lays the batch out and launches it when the model
@@ -489,7 +489,7 @@ class Engine:
             for g in range(n_groups):
                 table = np.asarray(tables[g][r], dtype=np.int32)
                 o = offsets["slots%d" % g][0] + row0
-                if self._group_stride[g] == 1:
+                if not self._group_of_blocks[g]:
                     a[o:o + n] = table[pos // ps] * ps + pos % ps
                 else:
                     a[o:o + n] = 0              # rows per block of tokens are addressed through the block table
@@ -796,7 +796,7 @@ class _DecodeGraph:
             slots.append(req.state_slot)
             for g in range(len(engine.groups)):
                 table = req.tables[g]
-                if engine._group_stride[g] == 1:
+                if not engine._group_of_blocks[g]:
                     a[o["slots%d" % g] + r] = table[p0 // ps] * ps + p0 % ps
                 key = (req.serial, len(table), req.first_live[g])
                 if self._row_keys[g][r] != key:

@@ -194,12 +194,12 @@ class Scheduler:
         decoding = [r for r in self.running if r.decoding]
         if decoding and len(decoding) <= budget:
             ps, reqs = self.cache.page_size, self.cache.requests
-            strides = [g.stride for g in self.cache.groups]
+            of_blocks = [g.of_blocks for g in self.cache.groups]
             need = [0] * ngroups
             for r in decoding:
                 e = reqs[r.task.id]
                 for g, table in enumerate(e.tables):
-                    pages = e.length // ps + 1 if strides[g] == 1 else self.cache._pages_for(e.length + 1, g)
+                    pages = self.cache._pages_for(e.length + 1, g) if of_blocks[g] else e.length // ps + 1
                     if len(table) < pages:
                         need[g] += pages - len(table)
             if self._fits(need, reserved):

@@ -136,6 +136,10 @@ _SIGNATURES = {
     "ic_rope_pairs_store": [_P, _I, _I, _P, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P],
     "ic_pool_blocks": [_P, _P, _P, _P, _I, _P, _I, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _P],
     "ic_attn_pooled_generic": [_P, _I, _P, _I, _I, _P, _P, _P, _P, _P, _I, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _I, _P],
+    "ic_attn_pooled_decode_supported": [_I, _I, _I],
+    "ic_attn_pooled_decode": [_P, _I, _P, _I, _I, _P, _P, _P, _P, _P, _I, _P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _I, _I, _P],
+    "ic_attn_pooled_prefill_supported": [_I, _I, _I],
+    "ic_attn_pooled_prefill": [_P, _I, _P, _I, _I, _P, _P, _P, _P, _P, _I, _P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _F, _I, _I, _P],
     "ic_moe_route": [_P, _I, _I, _I, _I, _I, _I, _P, _P, _P],
     "ic_moe_sort": [_P, _I, _I, _P, _P, _P, _P],
     "ic_moe_gather": [_P, _I, _I, _P, _P, _I, _I, _I, _P, _P],

@@ -1259,6 +1259,78 @@ def attention_pooled_generic(q, out, kcache, vcache, kpool, vpool, block_tables,
     return out
 
 
+def _pooled_common(q, out, kcache, vcache, kpool, vpool, block_tables, pool_tables, n_heads, n_kv_heads, key_dim, value_dim,
+                   page_size, window, block, bias, what):
+    T = q.shape[0]
+    _need(q.dim() == 2 and q.stride(1) == 1 and q.shape[1] == n_heads * key_dim and out.dtype == q.dtype and out.stride(1) == 1
+          and tuple(out.shape) == (T, n_heads * value_dim) and kcache.dtype == q.dtype, what + ": q/out layout")
+    _pooled_planes(kcache, vcache, kpool, vpool, n_kv_heads, key_dim, value_dim, page_size, what)
+    _need(block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.stride(1) == 1, what + ": block tables")
+    pooled = bool(window and block)
+    if pooled:
+        _need(pool_tables is not None and kpool is not None and pool_tables.dtype == torch.int32 and pool_tables.dim() == 2
+              and pool_tables.stride(1) == 1, what + ": the block means' planes and tables are missing")
+    _need(bias is None or (bias.dtype == torch.float32 and bias.numel() == n_heads and bias.is_contiguous()), what + ": bias")
+    return pooled
+
+
+def attention_pooled_decode_supported(dtype, key_dim: int, value_dim: int) -> bool:
+    return dtype in _DT and bool(get_lib().ic_attn_pooled_decode_supported(_DT[dtype], int(key_dim), int(value_dim)))
+
+
+def attention_pooled_decode(q, out, kcache, vcache, kpool, vpool, block_tables, pool_tables, tok_list, n_tok: int, token_req,
+                            positions, parts, bias, n_heads: int, n_kv_heads: int, key_dim: int, value_dim: int, page_size: int,
+                            scale: float, window: int, block: int, n_split: int = 1):
+    """As ``attention_pooled_generic`` for rows that are a request's single token (``tok_list``: their rows, None: rows
+    0 .. n_tok - 1), what each sees split ``n_split`` ways over blocks of threads; ``parts``: float32 scratch of
+    n_split * n_tok * heads * value_dim when n_split > 1."""
+    _dev(q, out, kcache, vcache, kpool, vpool, block_tables, pool_tables, tok_list, token_req, positions, parts, bias)
+    pooled = _pooled_common(q, out, kcache, vcache, kpool, vpool, block_tables, pool_tables, n_heads, n_kv_heads, key_dim,
+                            value_dim, page_size, window, block, bias, "attention_pooled_decode")
+    _i32(token_req, "token_req")
+    _i32(positions, "positions")
+    if tok_list is not None:
+        _i32(tok_list, "tok_list")
+        _need(tok_list.numel() >= n_tok, "attention_pooled_decode: tok_list")
+    else:
+        _need(n_tok <= q.shape[0], "attention_pooled_decode: more rows than q holds")
+    if n_split > 1:
+        _need(parts is not None and parts.dtype == torch.float32 and parts.is_contiguous()
+              and parts.numel() >= n_split * n_tok * n_heads * value_dim, "attention_pooled_decode: scratch for the splits")
+    check(get_lib().ic_attn_pooled_decode(q.data_ptr(), q.stride(0), out.data_ptr(), out.stride(0), dtype_code(q.dtype),
+                                          kcache.data_ptr(), vcache.data_ptr(), _ptr(kpool) if pooled else None,
+                                          _ptr(vpool) if pooled else None, block_tables.data_ptr(), block_tables.stride(0),
+                                          _ptr(pool_tables) if pooled else None, pool_tables.stride(0) if pooled else 0,
+                                          _ptr(tok_list), token_req.data_ptr(), positions.data_ptr(), _ptr(bias), _ptr(parts),
+                                          int(n_tok), n_heads, n_kv_heads, key_dim, value_dim, page_size, float(scale),
+                                          int(window or 0), int(block or 0), int(n_split), _stream()), "attention_pooled_decode")
+    return out
+
+
+def attention_pooled_prefill_supported(dtype, key_dim: int, value_dim: int, page_size: int = 16) -> bool:
+    return dtype in _DT and bool(get_lib().ic_attn_pooled_prefill_supported(_DT[dtype], int(key_dim), int(value_dim)))
+
+
+def attention_pooled_prefill(q, out, kcache, vcache, kpool, vpool, block_tables, pool_tables, tiles, n_tiles: int, bias,
+                             n_heads: int, n_kv_heads: int, key_dim: int, value_dim: int, page_size: int, scale: float,
+                             window: int, block: int):
+    """As ``attention_pooled_generic`` for prompt portions listed as tiles (int32 [n_tiles, 4]: request row, first token
+    row, rows <= 128, first position), on the matrix cores (bfloat16)."""
+    _dev(q, out, kcache, vcache, kpool, vpool, block_tables, pool_tables, tiles, bias)
+    pooled = _pooled_common(q, out, kcache, vcache, kpool, vpool, block_tables, pool_tables, n_heads, n_kv_heads, key_dim,
+                            value_dim, page_size, window, block, bias, "attention_pooled_prefill")
+    _need(tiles.dtype == torch.int32 and tiles.is_contiguous() and tiles.numel() >= 4 * n_tiles and tiles.data_ptr() % 16 == 0,
+          "attention_pooled_prefill: tiles must be int32 [n, 4], 16-byte aligned")
+    check(get_lib().ic_attn_pooled_prefill(q.data_ptr(), q.stride(0), out.data_ptr(), out.stride(0), dtype_code(q.dtype),
+                                           kcache.data_ptr(), vcache.data_ptr(), _ptr(kpool) if pooled else None,
+                                           _ptr(vpool) if pooled else None, block_tables.data_ptr(), block_tables.stride(0),
+                                           _ptr(pool_tables) if pooled else None, pool_tables.stride(0) if pooled else 0,
+                                           tiles.data_ptr(), int(n_tiles), _ptr(bias), n_heads, n_kv_heads, key_dim, value_dim,
+                                           page_size, float(scale), int(window or 0), int(block or 0), _stream()),
+          "attention_pooled_prefill")
+    return out
+
+
 # ---- routed experts (csrc/moe.hip) ----------------------------------------------------------------------------------------
 def moe_route(logits, top: int, ids, weights, mode: str = "sigmoid", renormalize: bool = False):
     """ids[t, k], weights[t, k]: the ``top`` experts with the largest scores of float32 ``logits`` [T, E] and their scores

@@ -117,8 +117,38 @@ class PooledAttention(Mixer):
         linear(out, self.w_o, y, rt.gemm_impl, ws=ctx.ws)
         return y
 
+    def portion_tile_rows(self):
+        return ops.attention_prefill_tile_rows()
+
     def _attend(self, q, out, ctx, cache, blocks):
-        ops.attention_pooled_generic(q, out, cache.k, cache.v, blocks.k if blocks else None, blocks.v if blocks else None,
-                                     cache.block_tables, blocks.block_tables if blocks else None, ctx.token_req, ctx.positions,
-                                     self.bias, self.nh, self.nkvh, self.dk, self.dv, ctx.page_size, self.scale, self.window,
-                                     self.block)
+        """Single-token rows go to the split kernel, prompt portions to the matrix-core kernel, where the sizes have one (and
+        the runtime does not ask for the general kernel alone); everything else to the general kernel."""
+        rt = self.runtime
+        planes = (cache.k, cache.v, blocks.k if blocks else None, blocks.v if blocks else None, cache.block_tables,
+                  blocks.block_tables if blocks else None)
+        tail = (self.bias, self.nh, self.nkvh, self.dk, self.dv, ctx.page_size, self.scale, self.window, self.block)
+        n_dec, n_tiles = ctx.n_decode_rows, ctx.n_prefill_tiles
+        tiled = rt.attention_impl == "auto" and n_dec + n_tiles > 0
+        use_dec = tiled and n_dec > 0 and ops.attention_pooled_decode_supported(rt.dtype, self.dk, self.dv)
+        use_pre = tiled and n_tiles > 0 and ops.attention_pooled_prefill_supported(rt.dtype, self.dk, self.dv, ctx.page_size)
+        if not tiled or not (use_dec or n_dec == 0) or not (use_pre or n_tiles == 0):
+            ops.attention_pooled_generic(q, out, *planes, ctx.token_req, ctx.positions, *tail)
+            return
+        if use_dec:
+            n_split = self._splits(ctx)
+            parts = ctx.ws.buffer("pooled_parts", (n_split * n_dec * self.nh * self.dv,), torch.float32) if n_split > 1 else None
+            ops.attention_pooled_decode(q, out, *planes, None if ctx.decode_rows_identity else ctx.decode_rows, n_dec,
+                                        ctx.token_req, ctx.positions, parts, *tail, n_split=n_split)
+        if use_pre:
+            ops.attention_pooled_prefill(q, out, *planes, ctx.prefill_tiles, n_tiles, *tail)
+
+    def _splits(self, ctx) -> int:
+        """Ways to split what single-token rows see: enough blocks of threads to fill the chip about twice, none with fewer
+        than 64 items; from the number of rows and the step's rounded key count, so that recorded steps split as eager ones."""
+        if ctx.fixed_decode_splits is not None:
+            return max(1, min(32, ctx.fixed_decode_splits))
+        most = ctx.max_context or 1
+        if self.window:
+            most = min(most, self.window) + (most // self.block if self.block else 0)
+        want = -(-2 * ctx.cu_count // max(1, ctx.n_decode_rows * self.nkvh))
+        return max(1, min(32, want, most // 64))

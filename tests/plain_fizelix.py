@@ -79,7 +79,7 @@ def rotate_pairs(x, positions, dims, base):
 
 
 # ---- attention over a window of tokens and the means of the blocks before it --------------------------------
-def visible(i, window, block, first_pooled=0):
+def visible(i, window, block):
     """What query position i sees: (token positions, block numbers).  Tokens j with 0 <= i - j < window; block b
     (positions b*block .. b*block + block - 1) once its last position is <= i - window."""
     tokens = [j for j in range(max(0, i - window + 1), i + 1)]
@@ -92,32 +92,44 @@ def visible(i, window, block, first_pooled=0):
     return tokens, blocks
 
 
-def pooled_sigmoid_attention(h, W, p, heads, kv_heads, dim, vdim, scale, window, block, rot_dims, rot_base, first=0):
-    """Weights are sigmoid(score + bias of the head) and are not normalised over the keys.  ``window`` None: all earlier
-    tokens and no blocks."""
+def seen_masks(T, window, block, first=0):
+    """([T, first + T] tokens seen, [T, blocks] blocks seen) for queries at positions first .. first + T - 1, from ``visible``."""
+    n_keys = first + T
+    n_blocks = n_keys // block if (block and window) else 0
+    tok = torch.zeros(T, n_keys, dtype=torch.bool)
+    blk = torch.zeros(T, n_blocks, dtype=torch.bool)
+    for t in range(T):
+        tokens, blocks = visible(first + t, window if window else n_keys + 1, block if window else 0)
+        tok[t, tokens] = True
+        blk[t, blocks] = True
+    return tok, blk
+
+
+def pooled_sigmoid_attention(h, W, p, heads, kv_heads, dim, vdim, scale, window, block, rot_dims, rot_base):
+    """Weights are sigmoid(score + bias of the head), for tokens and block means alike, and are not normalised over the
+    keys.  ``window`` None: all earlier tokens and no blocks.  Dense score matrices under the masks of ``seen_masks``."""
     T = h.shape[0]
-    positions = list(range(first, first + T))
+    positions = list(range(T))
     q = (h @ W[p + "q"].T).reshape(T, heads, dim)
     k = (h @ W[p + "k"].T).reshape(T, kv_heads, dim)
     v = (h @ W[p + "v"].T).reshape(T, kv_heads, vdim)
     if rot_dims:
         q, k = rotate_pairs(q, positions, rot_dims, rot_base), rotate_pairs(k, positions, rot_dims, rot_base)
+    tok, blk = seen_masks(T, window, block)
+    nb = blk.shape[1]
     per = heads // kv_heads
-    out = torch.zeros(T, heads, vdim, dtype=h.dtype)
-    n_blocks = T // block if (block and window) else 0
-    k_mean = [k[b * block:(b + 1) * block].mean(0) for b in range(n_blocks)]
-    v_mean = [v[b * block:(b + 1) * block].mean(0) for b in range(n_blocks)]
-    for i in range(T):
-        tokens, blocks = visible(i, window if window else T + 1, block if window else 0)
-        for hd in range(heads):
-            g = hd // per
-            acc = torch.zeros(vdim, dtype=h.dtype)
-            for j in tokens:
-                acc = acc + torch.sigmoid((q[i, hd] @ k[j, g]) * scale + W[p + "pb"][hd]) * v[j, g]
-            for b in blocks:
-                acc = acc + torch.sigmoid((q[i, hd] @ k_mean[b][g]) * scale + W[p + "pb"][hd]) * v_mean[b][g]
-            out[i, hd] = acc
-    return out.reshape(T, heads * vdim) @ W[p + "o"].T
+    out = []
+    for hd in range(heads):
+        g = hd // per
+        bias = W[p + "pb"][hd] if (p + "pb") in W else 0.0
+        w = torch.sigmoid((q[:, hd] @ k[:, g].T) * scale + bias) * tok
+        o = w @ v[:, g]
+        if nb:
+            k_mean = k[:nb * block, g].reshape(nb, block, dim).mean(1)
+            v_mean = v[:nb * block, g].reshape(nb, block, vdim).mean(1)
+            o = o + (torch.sigmoid((q[:, hd] @ k_mean.T) * scale + bias) * blk) @ v_mean
+        out.append(o)
+    return torch.cat(out, -1) @ W[p + "o"].T
 
 
 # ---- feed-forward -----------------------------------------------------------------------------------------
