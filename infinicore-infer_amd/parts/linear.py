@@ -21,6 +21,10 @@ torch.backends.cudnn.allow_tf32 = False
 # asks the same functions, so the two ways of issuing a step choose alike.
 TUNE_LIBRARY = False   # while True, every library product times the library's algorithms for its shape first
 TUNE_FLUSH = None      # while tuning: a tensor larger than the caches, overwritten before every timed launch
+# Products with a side (N or K) below this keep the library's first choice: timing compares speed alone, and among the
+# algorithms the library lists as taking a product with K = 64 one was met that is fastest and returns NaN.  Products this
+# thin (a router's, a low-rank gate's) have nothing to gain from the choice anyway.
+TUNE_MIN_SIDE = 256
 _tuned = set()
 
 
@@ -28,7 +32,7 @@ def _library(x, w, out, alpha: float = 1.0):
     """out = alpha * x w^T through the library, as the reference does for every product
     (inference_context.cpp:59-79): hipBLASLt called directly, torch's routine if it has no
     algorithm for the shape."""
-    if TUNE_LIBRARY:
+    if TUNE_LIBRARY and min(w.shape[0], w.shape[1]) >= TUNE_MIN_SIDE:
         key = (x.dtype, out.dtype, x.shape[0], w.shape[0], w.shape[1], x.stride(0), w.stride(0), out.stride(0))
         if key not in _tuned:
             _tuned.add(key)
