@@ -104,12 +104,14 @@ IC_EXPORT int ic_rope_pairs_store(const void* rows, int row_stride, int dtype, c
 // them) and their means go to row b of the request's block-mean cache.  grid (T, nkvh).
 // ---------------------------------------------------------------------------------------------
 template <typename T>
-__global__ void __launch_bounds__(64)
+__global__ void __launch_bounds__(256)
 pool_blocks_kernel(const T* __restrict__ kcache, const T* __restrict__ vcache, T* __restrict__ kpool, T* __restrict__ vpool,
                    const int* __restrict__ block_tables, int bt_stride, const int* __restrict__ pool_tables, int pt_stride,
                    const int* __restrict__ token_req, const int* __restrict__ positions, int P, int nkvh, int dk, int dv,
                    int page_size) {
-    const int t = blockIdx.x, g = blockIdx.y, lane = threadIdx.x;
+    // a wave a quarter of the block's rows (rows w, w + 4, ..), a lane a column; the four shares meet in LDS
+    __shared__ float part[4][2 * kPoolMaxDim];
+    const int t = blockIdx.x, g = blockIdx.y, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int p = positions[t];
     if ((p + 1) % P != 0) return;
     const int b = (p + 1) / P - 1;
@@ -121,7 +123,14 @@ pool_blocks_kernel(const T* __restrict__ kcache, const T* __restrict__ vcache, T
         const int c = key ? d : d - dk, w = key ? dk : dv;
         const T* plane = key ? kcache : vcache;
         float s = 0.f;
-        for (int j = 0; j < P; ++j) s += to_f32(plane[cache_row(bt, b * P + j, page_size, nkvh, g) * w + c]);
+        for (int j = wave; j < P; j += 4) s += to_f32(plane[cache_row(bt, b * P + j, page_size, nkvh, g) * w + c]);
+        part[wave][d] = s;
+    }
+    __syncthreads();
+    for (int d = threadIdx.x; d < dk + dv; d += 256) {
+        const bool key = d < dk;
+        const int c = key ? d : d - dk, w = key ? dk : dv;
+        const float s = (part[0][d] + part[1][d]) + (part[2][d] + part[3][d]);
         (key ? kpool : vpool)[orow * w + c] = from_f32<T>(s / (float)P);
     }
 }
@@ -131,8 +140,8 @@ IC_EXPORT int ic_pool_blocks(const void* kcache, const void* vcache, void* kpool
                              const int* token_req, const int* positions, int T, int P, int nkvh, int dk, int dv,
                              int page_size, hipStream_t stream) {
     if (T <= 0) return IC_OK;
-    if (P <= 0 || nkvh <= 0 || nkvh > 65535 || dk <= 0 || dv <= 0 || page_size <= 0) return IC_ERR_ARG;
-    dim3 grid((unsigned)T, (unsigned)nkvh), block(64);
+    if (P <= 0 || nkvh <= 0 || nkvh > 65535 || dk <= 0 || dv <= 0 || dk > kPoolMaxDim || dv > kPoolMaxDim || page_size <= 0) return IC_ERR_ARG;
+    dim3 grid((unsigned)T, (unsigned)nkvh), block(256);
     if (dtype == IC_F32)
         hipLaunchKernelGGL(pool_blocks_kernel<float>, grid, block, 0, stream, (const float*)kcache, (const float*)vcache,
                            (float*)kpool, (float*)vpool, block_tables, bt_stride, pool_tables, pt_stride, token_req, positions,
@@ -399,7 +408,7 @@ __global__ void __launch_bounds__(256)
 attn_pooled_merge_kernel(const float* __restrict__ parts, const int* __restrict__ tok_list, T* __restrict__ out, int out_stride,
                          int n_tok, int width, int nsplit) {
     const int ti = blockIdx.x, t = tok_list ? tok_list[ti] : ti;
-    for (int i = threadIdx.x; i < width; i += blockDim.x) {
+    for (int i = blockIdx.y * blockDim.x + threadIdx.x; i < width; i += gridDim.y * blockDim.x) {
         float v = 0.f;
         for (int s = 0; s < nsplit; ++s) v += parts[((size_t)s * n_tok + ti) * width + i];
         out[(size_t)t * out_stride + i] = from_f32<T>(v);
@@ -441,10 +450,10 @@ IC_EXPORT int ic_attn_pooled_decode(const void* q, int q_stride, void* out, int 
     int st = ic_launch_status();
     if (st != IC_OK || nsplit == 1) return st;
     if (dtype == IC_F32)
-        hipLaunchKernelGGL(attn_pooled_merge_kernel<float>, dim3(n_tok), dim3(256), 0, stream, parts, tok_list, (float*)out,
+        hipLaunchKernelGGL(attn_pooled_merge_kernel<float>, dim3(n_tok, (nh * dv + 255) / 256), dim3(256), 0, stream, parts, tok_list, (float*)out,
                            out_stride, n_tok, nh * dv, nsplit);
     else
-        hipLaunchKernelGGL(attn_pooled_merge_kernel<bf16>, dim3(n_tok), dim3(256), 0, stream, parts, tok_list, (bf16*)out,
+        hipLaunchKernelGGL(attn_pooled_merge_kernel<bf16>, dim3(n_tok, (nh * dv + 255) / 256), dim3(256), 0, stream, parts, tok_list, (bf16*)out,
                            out_stride, n_tok, nh * dv, nsplit);
     return ic_launch_status();
 }

@@ -236,10 +236,87 @@ moe_expert_product_kernel(const T* __restrict__ a, int a_stride, const T* __rest
     }
 }
 
+
+// ---------------------------------------------------------------------------------------------
+// The same product on the matrix cores (bfloat16, N a multiple of 16, K of 32).  Grid (N / 16, experts), four waves:
+// a block owns 16 output columns of one expert (with GLU: 16 gate rows and the matching 16 up rows); its waves take
+// the k-steps of 32 in turn, so that together they read 256 consecutive bytes of every weight row at a time.  Lane
+// (r = l % 16, kq = l / 16) loads 16 bytes W[c0 + r][k0 + 8 kq ..] and the matching 16 bytes of token row r of the
+// chunk, and feeds them to one v_mfma_f32_16x16x32_bf16 as A and B operands (D[i = 4 (l / 16) + e][j = l % 16]:
+// column c0 + i of token row j).  The waves' sums meet in LDS.  An expert's rows are taken 16 at a time; the token
+// rows are few and come out of the caches, the weights are streamed with loads the caches do not keep.
+// ---------------------------------------------------------------------------------------------
+typedef __bf16 moe_v8b __attribute__((ext_vector_type(8)));
+typedef float moe_v4f __attribute__((ext_vector_type(4)));
+
+template <bool GLU>
+__global__ void __launch_bounds__(256)
+moe_expert_product_mfma_kernel(const uint16_t* __restrict__ a, int a_stride, const uint16_t* __restrict__ w,
+                               long long w_expert_stride, const int* __restrict__ offsets, uint16_t* __restrict__ out,
+                               int out_stride, int N, int K) {
+    __shared__ float sums[4][GLU ? 2 : 1][16][17];
+    const int e = blockIdx.y, c0 = blockIdx.x * 16;
+    const int r0 = offsets[e], r1 = offsets[e + 1];
+    if (r0 >= r1) return;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int r = lane & 15, kq = lane >> 4;
+    const uint16_t* w1 = w + (size_t)e * w_expert_stride + (size_t)(c0 + r) * K + 8 * kq;
+    const uint16_t* w2 = w1 + (size_t)N * K;
+    const int steps = K / 32;
+    for (int rb = r0; rb < r1; rb += 16) {
+        const int row = rb + r;
+        const bool row_ok = row < r1;
+        const uint16_t* ar = a + (size_t)(row_ok ? row : r1 - 1) * a_stride + 8 * kq;
+        moe_v4f acc = moe_v4f{0.f, 0.f, 0.f, 0.f}, acc2 = acc;
+#pragma unroll 4
+        for (int s = wave; s < steps; s += 4) {
+            const uint4 wa = load_stream16(w1 + 32 * s);
+            uint4 xa = *reinterpret_cast<const uint4*>(ar + 32 * s);
+            if (!row_ok) xa = uint4{0u, 0u, 0u, 0u};
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(moe_v8b, wa), __builtin_bit_cast(moe_v8b, xa), acc, 0, 0, 0);
+            if (GLU) {
+                const uint4 wb = load_stream16(w2 + 32 * s);
+                acc2 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(moe_v8b, wb), __builtin_bit_cast(moe_v8b, xa), acc2, 0, 0, 0);
+            }
+        }
+        __syncthreads();                                   // the chunk before has been summed
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            sums[wave][0][4 * kq + i][r] = acc[i];
+            if (GLU) sums[wave][GLU ? 1 : 0][4 * kq + i][r] = acc2[i];
+        }
+        __syncthreads();
+        {
+            const int col = tid >> 4, j = tid & 15;        // 256 threads: 16 columns x 16 token rows
+            if (rb + j < r1) {
+                float v = sums[0][0][col][j] + sums[1][0][col][j] + sums[2][0][col][j] + sums[3][0][col][j];
+                if (GLU) {
+                    const float u2 = sums[0][GLU ? 1 : 0][col][j] + sums[1][GLU ? 1 : 0][col][j] + sums[2][GLU ? 1 : 0][col][j] + sums[3][GLU ? 1 : 0][col][j];
+                    // gate and up are rounded to bfloat16 first, as a product kernel followed by the gated unit's kernel leaves them
+                    const float g = bf16_bits_to_f32(f32_to_bf16_bits(v)), u = bf16_bits_to_f32(f32_to_bf16_bits(u2));
+                    v = u * (g / (1.0f + expf(-g)));
+                }
+                out[(size_t)(rb + j) * out_stride + c0 + col] = f32_to_bf16_bits(v);
+            }
+        }
+    }
+}
+
 IC_EXPORT int ic_moe_expert_product(const void* a, int a_stride, const void* w, long long w_expert_stride, int dtype,
                                     const int* offsets, void* out, int out_stride, int E, int N, int K, int glu,
                                     int compute_units, hipStream_t stream) {
     if (E <= 0 || E > 65535 || N <= 0 || K <= 0) return IC_ERR_ARG;
+    if (dtype == IC_BF16 && N % 16 == 0 && K % 32 == 0 && (w_expert_stride % 8) == 0 && (a_stride % 8) == 0 &&
+        ((uintptr_t)w % 16) == 0 && ((uintptr_t)a % 16) == 0 && N / 16 <= 0x7fffffff / 2) {
+        dim3 grid((unsigned)(N / 16), (unsigned)E), block(256);
+        if (glu)
+            hipLaunchKernelGGL(moe_expert_product_mfma_kernel<true>, grid, block, 0, stream, (const uint16_t*)a, a_stride,
+                               (const uint16_t*)w, w_expert_stride, offsets, (uint16_t*)out, out_stride, N, K);
+        else
+            hipLaunchKernelGGL(moe_expert_product_mfma_kernel<false>, grid, block, 0, stream, (const uint16_t*)a, a_stride,
+                               (const uint16_t*)w, w_expert_stride, offsets, (uint16_t*)out, out_stride, N, K);
+        return ic_launch_status();
+    }
     int rc = 8;
     while (rc > 1 && (size_t)rc * K * sizeof(float) > 64 * 1024) rc >>= 1;
     const size_t lds = (size_t)rc * K * sizeof(float);

@@ -492,6 +492,8 @@ IC_EXPORT int ic_activation(const void* in, void* out, int dtype, long long n, i
 //   v = y[t] * sigmoid(g[t] + gb);  x[t] += v * rsqrt(mean(v^2) + eps) * w;  copy[t] = x[t] in the compute dtype.
 // g null: no gate (the kernel is then the plain norm into the stream).  One block per row.
 // ---------------------------------------------------------------------------------------------
+constexpr int kGnKeep = 16;       // gated values a thread keeps between the two passes (rows up to 256 * 16 wide)
+
 template <typename TY, typename TC>
 __global__ void __launch_bounds__(256)
 gated_norm_into_stream_kernel(const TY* __restrict__ y, const TY* __restrict__ g, int g_stride, const float* __restrict__ gb,
@@ -500,19 +502,37 @@ gated_norm_into_stream_kernel(const TY* __restrict__ y, const TY* __restrict__ g
     const int t = blockIdx.x;
     const TY* yr = y + (size_t)t * d;
     const TY* gr = g ? g + (size_t)t * g_stride : nullptr;
-    float ss = 0.f;
-    for (int i = threadIdx.x; i < d; i += blockDim.x) {
+    auto gated = [&](int i) {
         float v = to_f32(yr[i]);
         if (gr) v *= 1.0f / (1.0f + expf(-(to_f32(gr[i]) + (gb ? gb[i] : 0.f))));
+        return v;
+    };
+    float keep[kGnKeep];
+    float ss = 0.f;
+#pragma unroll
+    for (int n = 0; n < kGnKeep; ++n) {
+        const int i = threadIdx.x + n * 256;
+        keep[n] = i < d ? gated(i) : 0.f;
+        ss += keep[n] * keep[n];
+    }
+    for (int i = threadIdx.x + kGnKeep * 256; i < d; i += 256) {
+        const float v = gated(i);
         ss += v * v;
     }
     ss = block_sum(ss, red);
     const float r = 1.0f / sqrtf(ss / (float)d + eps);
     float* xr = x + (size_t)t * d;
-    for (int i = threadIdx.x; i < d; i += blockDim.x) {
-        float v = to_f32(yr[i]);
-        if (gr) v *= 1.0f / (1.0f + expf(-(to_f32(gr[i]) + (gb ? gb[i] : 0.f))));
-        const float s = xr[i] + v * r * w[i];
+#pragma unroll
+    for (int n = 0; n < kGnKeep; ++n) {
+        const int i = threadIdx.x + n * 256;
+        if (i < d) {
+            const float s = xr[i] + keep[n] * r * w[i];
+            xr[i] = s;
+            if (copy) copy[(size_t)t * d + i] = from_f32<TC>(s);
+        }
+    }
+    for (int i = threadIdx.x + kGnKeep * 256; i < d; i += 256) {
+        const float s = xr[i] + gated(i) * r * w[i];
         xr[i] = s;
         if (copy) copy[(size_t)t * d + i] = from_f32<TC>(s);
     }

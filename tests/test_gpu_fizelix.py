@@ -632,14 +632,16 @@ def test_routed_experts_kernels(dtype, T, E, top, d, ff, mode, renorm, on_input)
     assert torch.allclose(out.cpu().double(), want_out, atol=tol * max(1.0, float(want_out.abs().max())))
 
 
+@pytest.mark.parametrize("d,ff", [(48, 40), (64, 32)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_routed_experts_part_for_few_and_many_rows(dtype):
-    """The part with few rows (no integer leaves the device) and with many (one library product per expert) against the plain
-    feed-forward; the weight on the expert's input, a shared expert, four experts of six."""
+def test_routed_experts_part_for_few_and_many_rows(dtype, d, ff):
+    """The part with few rows (no integer leaves the device; sizes the matrix-core product takes and sizes it does not, more
+    than sixteen rows an expert) and with many (one library product per expert) against the plain feed-forward; the weight on
+    the expert's input, a shared expert, four experts of six."""
     from infinicore_infer_amd.engine.context import StepContext, Workspace
     from infinicore_infer_amd.parts import Runtime
     from infinicore_infer_amd.parts.routed_experts import RoutedExperts
-    d, E, top, ff, sh = 48, 6, 4, 40, 56
+    E, top, sh = 6, 4, 56
     cfg = {"vocab": 8, "width": d, "layers": [{"type": "attention", "mixer": {"heads": 1, "dim": 8}, "mlp": _moe(E, top, ff, sh)}]}
     W = {k[len("l0.mlp."):]: v for k, v in P.random_weights(cfg, 5).items() if k.startswith("l0.mlp.")}
     part = RoutedExperts("", Runtime(dtype, "cuda"), d, E, top, ff, sh)
