@@ -99,56 +99,60 @@ IC_EXPORT int ic_rope_pairs_store(const void* rows, int row_stride, int dtype, c
 }
 
 // ---------------------------------------------------------------------------------------------
-// The mean key and value of every block that this step completes: a token at position p with (p + 1) % P == 0
-// ends block b = (p + 1) / P - 1; its P keys and values are read back from the token cache (as the cache holds
-// them) and their means go to row b of the request's block-mean cache.  grid (T, nkvh).
+// The mean key and value of every block that this step completes.  A request's portion at positions p0 .. p0 + n - 1
+// completes the blocks b = p0 / P, p0 / P + 1, .. with (b + 1) P <= p0 + n; their P keys and values are read back from
+// the token cache (as the cache holds them) and their means go to row b of the request's block-mean cache.
+// grid (most blocks a request can complete, kv heads, requests); req_rows: first token row of every request, then T.
 // ---------------------------------------------------------------------------------------------
 template <typename T>
 __global__ void __launch_bounds__(256)
 pool_blocks_kernel(const T* __restrict__ kcache, const T* __restrict__ vcache, T* __restrict__ kpool, T* __restrict__ vpool,
                    const int* __restrict__ block_tables, int bt_stride, const int* __restrict__ pool_tables, int pt_stride,
-                   const int* __restrict__ token_req, const int* __restrict__ positions, int P, int nkvh, int dk, int dv,
+                   const int* __restrict__ req_rows, const int* __restrict__ positions, int P, int nkvh, int dk, int dv,
                    int page_size) {
-    // a wave a quarter of the block's rows (rows w, w + 4, ..), a lane a column; the four shares meet in LDS
-    __shared__ float part[4][2 * kPoolMaxDim];
-    const int t = blockIdx.x, g = blockIdx.y, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int p = positions[t];
-    if ((p + 1) % P != 0) return;
-    const int b = (p + 1) / P - 1;
-    const int* bt = block_tables + (size_t)token_req[t] * bt_stride;
-    const int* pt = pool_tables + (size_t)token_req[t] * pt_stride;
+    // a thread a column; the block's rows eight at a time, so that eight loads are in flight
+    const int r = blockIdx.z, g = blockIdx.y;
+    const int row0 = req_rows[r], n = req_rows[r + 1] - row0;
+    if (n <= 0) return;
+    const int p0 = positions[row0];
+    const int b = p0 / P + (int)blockIdx.x;
+    if ((long long)(b + 1) * P > (long long)p0 + n) return;
+    const int* bt = block_tables + (size_t)r * bt_stride;
+    const int* pt = pool_tables + (size_t)r * pt_stride;
     const long long orow = cache_row(pt, b, page_size, nkvh, g);
-    for (int d = lane; d < dk + dv; d += 64) {
+    for (int d = threadIdx.x; d < dk + dv; d += 256) {
         const bool key = d < dk;
         const int c = key ? d : d - dk, w = key ? dk : dv;
         const T* plane = key ? kcache : vcache;
         float s = 0.f;
-        for (int j = wave; j < P; j += 4) s += to_f32(plane[cache_row(bt, b * P + j, page_size, nkvh, g) * w + c]);
-        part[wave][d] = s;
-    }
-    __syncthreads();
-    for (int d = threadIdx.x; d < dk + dv; d += 256) {
-        const bool key = d < dk;
-        const int c = key ? d : d - dk, w = key ? dk : dv;
-        const float s = (part[0][d] + part[1][d]) + (part[2][d] + part[3][d]);
+        for (int j0 = 0; j0 < P; j0 += 8) {
+            float v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const int j = min(j0 + u, P - 1);
+                v[u] = to_f32(plane[cache_row(bt, b * P + j, page_size, nkvh, g) * w + c]);
+            }
+#pragma unroll
+            for (int u = 0; u < 8; ++u) s += (j0 + u < P) ? v[u] : 0.f;
+        }
         (key ? kpool : vpool)[orow * w + c] = from_f32<T>(s / (float)P);
     }
 }
 
 IC_EXPORT int ic_pool_blocks(const void* kcache, const void* vcache, void* kpool, void* vpool, int dtype,
                              const int* block_tables, int bt_stride, const int* pool_tables, int pt_stride,
-                             const int* token_req, const int* positions, int T, int P, int nkvh, int dk, int dv,
-                             int page_size, hipStream_t stream) {
-    if (T <= 0) return IC_OK;
-    if (P <= 0 || nkvh <= 0 || nkvh > 65535 || dk <= 0 || dv <= 0 || dk > kPoolMaxDim || dv > kPoolMaxDim || page_size <= 0) return IC_ERR_ARG;
-    dim3 grid((unsigned)T, (unsigned)nkvh), block(256);
+                             const int* req_rows, const int* positions, int n_requests, int most_blocks, int P, int nkvh,
+                             int dk, int dv, int page_size, hipStream_t stream) {
+    if (n_requests <= 0 || most_blocks <= 0) return IC_OK;
+    if (P <= 0 || nkvh <= 0 || nkvh > 65535 || n_requests > 65535 || dk <= 0 || dv <= 0 || page_size <= 0) return IC_ERR_ARG;
+    dim3 grid((unsigned)most_blocks, (unsigned)nkvh, (unsigned)n_requests), block(256);
     if (dtype == IC_F32)
         hipLaunchKernelGGL(pool_blocks_kernel<float>, grid, block, 0, stream, (const float*)kcache, (const float*)vcache,
-                           (float*)kpool, (float*)vpool, block_tables, bt_stride, pool_tables, pt_stride, token_req, positions,
+                           (float*)kpool, (float*)vpool, block_tables, bt_stride, pool_tables, pt_stride, req_rows, positions,
                            P, nkvh, dk, dv, page_size);
     else if (dtype == IC_BF16)
         hipLaunchKernelGGL(pool_blocks_kernel<bf16>, grid, block, 0, stream, (const bf16*)kcache, (const bf16*)vcache,
-                           (bf16*)kpool, (bf16*)vpool, block_tables, bt_stride, pool_tables, pt_stride, token_req, positions,
+                           (bf16*)kpool, (bf16*)vpool, block_tables, bt_stride, pool_tables, pt_stride, req_rows, positions,
                            P, nkvh, dk, dv, page_size);
     else
         return IC_ERR_UNSUPPORTED;
@@ -277,19 +281,22 @@ template <typename T> struct PoolVec;
 template <> struct PoolVec<float> {
     static constexpr int N = 4;
     __device__ static void load(const float* p, float* o) {
-        const float4 v = *reinterpret_cast<const float4*>(p);
-        o[0] = v.x; o[1] = v.y; o[2] = v.z; o[3] = v.w;
+        const uint4 v = load_stream16(p);
+        o[0] = __uint_as_float(v.x); o[1] = __uint_as_float(v.y); o[2] = __uint_as_float(v.z); o[3] = __uint_as_float(v.w);
     }
+    __device__ static float sigmoid(float z) { return 1.0f / (1.0f + expf(-z)); }
 };
 template <> struct PoolVec<bf16> {
     static constexpr int N = 8;
     __device__ static void load(const bf16* p, float* o) {
-        const uint4 v = *reinterpret_cast<const uint4*>(p);
+        const uint4 v = load_stream16(p);
         o[0] = __uint_as_float(v.x << 16); o[1] = __uint_as_float(v.x & 0xffff0000u);
         o[2] = __uint_as_float(v.y << 16); o[3] = __uint_as_float(v.y & 0xffff0000u);
         o[4] = __uint_as_float(v.z << 16); o[5] = __uint_as_float(v.z & 0xffff0000u);
         o[6] = __uint_as_float(v.w << 16); o[7] = __uint_as_float(v.w & 0xffff0000u);
     }
+    // the hardware's exp2 and reciprocal (each good to an ulp): for results that are rounded to bfloat16
+    __device__ static float sigmoid(float z) { return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * z)); }
 };
 
 constexpr int kPdHeads = 4;      // query heads served per walk
@@ -362,7 +369,7 @@ attn_pooled_decode_kernel(const T* __restrict__ q, int q_stride, const T* __rest
 #pragma unroll
                 for (int j = 0; j < VEC; ++j) d += kf[j] * qr[g][j];
                 d = group_sum<LPK>(d);
-                const float p = sigmoid_acc(d * scale + hb[g]);
+                const float p = PoolVec<T>::sigmoid(d * scale + hb[g]);
 #pragma unroll
                 for (int n = 0; n < NP; ++n)
 #pragma unroll

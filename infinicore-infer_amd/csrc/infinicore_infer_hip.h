@@ -154,8 +154,9 @@ int ic_matmul_tune(const void* A, int a_dtype, const void* W, void* C, int c_dty
 // Adjacent pairs (2i, 2i+1) of the first rot_dims entries of every q and k head turn by position * f_i (freq: float32
 // [2, rot_dims / 2], the rounded frequency and what the rounding left); q -> q_out, k and v -> the cache at slots (null: q only).
 int ic_rope_pairs_store(const void* rows, int row_stride, int dtype, const int* positions, const float* freq, int rot_dims, void* q_out, void* kcache, void* vcache, const int* slots, int T, int nh, int nkvh, int dk, int dv, int page_size, hipStream_t stream);
-// Means of the blocks of P tokens that the step's tokens complete, from the token cache into row b of the block-mean cache.
-int ic_pool_blocks(const void* kcache, const void* vcache, void* kpool, void* vpool, int dtype, const int* block_tables, int bt_stride, const int* pool_tables, int pt_stride, const int* token_req, const int* positions, int T, int P, int nkvh, int dk, int dv, int page_size, hipStream_t stream);
+// Means of the blocks of P tokens that the step's portions complete (req_rows: first token row of every request, then T;
+// most_blocks: an upper bound on the blocks one request completes), from the token cache into row b of the block-mean cache.
+int ic_pool_blocks(const void* kcache, const void* vcache, void* kpool, void* vpool, int dtype, const int* block_tables, int bt_stride, const int* pool_tables, int pt_stride, const int* req_rows, const int* positions, int n_requests, int most_blocks, int P, int nkvh, int dk, int dv, int page_size, hipStream_t stream);
 // out_i = sum over seen tokens and blocks of sigmoid(scale q.k + bias[h]) v; any sizes up to 512, float32 or bfloat16.
 int ic_attn_pooled_generic(const void* q, int q_stride, void* out, int out_stride, int dtype, const void* kcache, const void* vcache, const void* kpool, const void* vpool, const int* block_tables, int bt_stride, const int* pool_tables, int pt_stride, const int* token_req, const int* positions, const float* bias, int T, int nh, int nkvh, int dk, int dv, int page_size, float scale, int window, int P, hipStream_t stream);
 // Single tokens, split over what they see (key and value sizes 64 or 128; parts: float32 [nsplit, n_tok, nh, dv] when nsplit > 1).

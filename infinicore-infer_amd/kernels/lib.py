@@ -134,7 +134,7 @@ _SIGNATURES = {
     "ic_latent_gather": [_P, _I, _P, _I, _I, _I, _I, _I, _P, _P, _P],
     "ic_latent_softmax": [_P, _I, _P, _I, _I, _I, _I, _I, _I, _F, _P],
     "ic_rope_pairs_store": [_P, _I, _I, _P, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P],
-    "ic_pool_blocks": [_P, _P, _P, _P, _I, _P, _I, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _P],
+    "ic_pool_blocks": [_P, _P, _P, _P, _I, _P, _I, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P],
     "ic_attn_pooled_generic": [_P, _I, _P, _I, _I, _P, _P, _P, _P, _P, _I, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _I, _P],
     "ic_attn_pooled_decode_supported": [_I, _I, _I],
     "ic_attn_pooled_decode": [_P, _I, _P, _I, _I, _P, _P, _P, _P, _P, _I, _P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _I, _I, _P],

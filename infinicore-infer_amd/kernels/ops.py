@@ -1215,20 +1215,21 @@ def _pooled_planes(kcache, vcache, kpool, vpool, n_kv_heads, key_dim, value_dim,
               and tuple(v.shape[1:]) == (n_kv_heads, page_size, value_dim) and k.shape[0] == v.shape[0], what + ": cache planes")
 
 
-def pool_blocks(kcache, vcache, kpool, vpool, block_tables, pool_tables, token_req, positions, block: int, n_kv_heads: int,
-                key_dim: int, value_dim: int, page_size: int):
-    """For every token of the step that ends a block of ``block`` tokens (position p with (p + 1) % block == 0): the means of
-    the block's keys and values, read from the token cache, into row (p + 1) / block - 1 of the request's block-mean cache."""
-    _dev(kcache, vcache, kpool, vpool, block_tables, pool_tables, token_req, positions)
+def pool_blocks(kcache, vcache, kpool, vpool, block_tables, pool_tables, req_rows, positions, n_requests: int, most_tokens: int,
+                block: int, n_kv_heads: int, key_dim: int, value_dim: int, page_size: int):
+    """For every block of ``block`` tokens that a request's portion completes (its last position lies in the portion): the
+    means of the block's keys and values, read from the token cache, into row b of the request's block-mean cache.
+    ``req_rows``: first token row of every request, then T; ``most_tokens``: the longest portion of the step."""
+    _dev(kcache, vcache, kpool, vpool, block_tables, pool_tables, req_rows, positions)
     _pooled_planes(kcache, vcache, kpool, vpool, n_kv_heads, key_dim, value_dim, page_size, "pool_blocks")
-    for t, n in ((block_tables, "block_tables"), (pool_tables, "pool_tables"), (token_req, "token_req"), (positions, "positions")):
+    for t, n in ((block_tables, "block_tables"), (pool_tables, "pool_tables"), (req_rows, "req_rows"), (positions, "positions")):
         _need(t.dtype == torch.int32 and t.stride(-1) == 1, "pool_blocks: %s must be int32" % n)
-    T = positions.numel()
-    _need(block > 0 and token_req.numel() >= T and block_tables.dim() == 2 and pool_tables.dim() == 2, "pool_blocks: lists")
+    _need(block > 0 and req_rows.numel() >= n_requests + 1 and block_tables.dim() == 2 and pool_tables.dim() == 2
+          and block_tables.shape[0] >= n_requests and pool_tables.shape[0] >= n_requests and most_tokens >= 1, "pool_blocks: lists")
     check(get_lib().ic_pool_blocks(kcache.data_ptr(), vcache.data_ptr(), kpool.data_ptr(), vpool.data_ptr(), dtype_code(kcache.dtype),
                                    block_tables.data_ptr(), block_tables.stride(0), pool_tables.data_ptr(), pool_tables.stride(0),
-                                   token_req.data_ptr(), positions.data_ptr(), T, int(block), n_kv_heads, key_dim, value_dim,
-                                   page_size, _stream()), "pool_blocks")
+                                   req_rows.data_ptr(), positions.data_ptr(), int(n_requests), int(most_tokens) // int(block) + 1,
+                                   int(block), n_kv_heads, key_dim, value_dim, page_size, _stream()), "pool_blocks")
 
 
 def attention_pooled_generic(q, out, kcache, vcache, kpool, vpool, block_tables, pool_tables, token_req, positions, bias,

@@ -109,8 +109,8 @@ class PooledAttention(Mixer):
         if self.block and blocks is None:
             raise RuntimeError("pooled attention %s: the cache holds no rows for the blocks' means" % self.name)
         if blocks is not None and cache.writes:
-            ops.pool_blocks(cache.k, cache.v, blocks.k, blocks.v, cache.block_tables, blocks.block_tables, ctx.token_req,
-                            ctx.positions, self.block, self.nkvh, self.dk, self.dv, ctx.page_size)
+            ops.pool_blocks(cache.k, cache.v, blocks.k, blocks.v, cache.block_tables, blocks.block_tables, ctx.req_rows,
+                            ctx.positions, ctx.R, max(ctx.req_len), self.block, self.nkvh, self.dk, self.dv, ctx.page_size)
         out = ctx.ws.buffer("pooled_out", (T, self.na), rt.dtype)
         self._attend(q, out, ctx, cache, blocks)
         y = ctx.ws.buffer("mixer_out", (T, self.hidden_size), rt.dtype)
@@ -143,12 +143,12 @@ class PooledAttention(Mixer):
             ops.attention_pooled_prefill(q, out, *planes, ctx.prefill_tiles, n_tiles, *tail)
 
     def _splits(self, ctx) -> int:
-        """Ways to split what single-token rows see: enough blocks of threads to fill the chip about twice, none with fewer
+        """Ways to split what single-token rows see: enough blocks of threads to fill the chip about four times, none with fewer
         than 64 items; from the number of rows and the step's rounded key count, so that recorded steps split as eager ones."""
         if ctx.fixed_decode_splits is not None:
             return max(1, min(32, ctx.fixed_decode_splits))
         most = ctx.max_context or 1
         if self.window:
             most = min(most, self.window) + (most // self.block if self.block else 0)
-        want = -(-2 * ctx.cu_count // max(1, ctx.n_decode_rows * self.nkvh))
+        want = -(-4 * ctx.cu_count // max(1, ctx.n_decode_rows * self.nkvh))
         return max(1, min(32, want, most // 64))

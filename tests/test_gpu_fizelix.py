@@ -464,10 +464,13 @@ def test_means_of_the_blocks_a_step_completes(dtype, G, dk, dv, block, page):
     steps = [[(0, 0, 150), (1, 0, 3), (2, 0, 1)], [(1, 3, block), (2, 1, 2)], [(1, 3 + block, 1)], [(1, 4 + block, 70 - 4 - block), (2, 3, 6)]]
     done = {0: 0, 1: 0, 2: 0}
     for step in steps:
-        token_req = sum(([i] * n for i, (r, p0, n) in enumerate(step)), [])
         positions = sum((list(range(p0, p0 + n)) for r, p0, n in step), [])
+        req_rows = [0]
+        for _, _, n in step:
+            req_rows.append(req_rows[-1] + n)
         rows = torch.tensor([r for r, _, _ in step])
-        ops.pool_blocks(kc, vc, kp, vp, bt[rows].contiguous(), pt[rows].contiguous(), _i32(token_req), _i32(positions), block, G, dk, dv, page)
+        ops.pool_blocks(kc, vc, kp, vp, bt[rows].contiguous(), pt[rows].contiguous(), _i32(req_rows), _i32(positions), len(step),
+                        max(n for _, _, n in step), block, G, dk, dv, page)
         for r, p0, n in step:
             done[r] = (p0 + n) // block
         for r in range(3):
