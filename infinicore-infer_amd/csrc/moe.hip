@@ -243,7 +243,8 @@ moe_expert_product_kernel(const T* __restrict__ a, int a_stride, const T* __rest
 // the k-steps of 32 in turn, so that together they read 256 consecutive bytes of every weight row at a time.  Lane
 // (r = l % 16, kq = l / 16) loads 16 bytes W[c0 + r][k0 + 8 kq ..] and the matching 16 bytes of token row r of the
 // chunk, and feeds them to one v_mfma_f32_16x16x32_bf16 as A and B operands (D[i = 4 (l / 16) + e][j = l % 16]:
-// column c0 + i of token row j).  The waves' sums meet in LDS.  An expert's rows are taken 16 at a time; the token
+// column c0 + i of token row j).  The waves' sums meet in LDS.  An expert's rows are taken 32 at a time (two tiles of 16 per
+// pass over the weights; the second only where the expert has that many rows); the token
 // rows are few and come out of the caches, the weights are streamed with loads the caches do not keep.
 // ---------------------------------------------------------------------------------------------
 typedef __bf16 moe_v8b __attribute__((ext_vector_type(8)));
@@ -254,7 +255,9 @@ __global__ void __launch_bounds__(256)
 moe_expert_product_mfma_kernel(const uint16_t* __restrict__ a, int a_stride, const uint16_t* __restrict__ w,
                                long long w_expert_stride, const int* __restrict__ offsets, uint16_t* __restrict__ out,
                                int out_stride, int N, int K) {
-    __shared__ float sums[4][GLU ? 2 : 1][16][17];
+    constexpr int NW = GLU ? 2 : 1;                       // weight rows per column: gate and up, or one
+    constexpr int MT = 2;                                 // tiles of 16 token rows per pass over the weights
+    __shared__ float sums[4][MT][NW][16][17];
     const int e = blockIdx.y, c0 = blockIdx.x * 16;
     const int r0 = offsets[e], r1 = offsets[e + 1];
     if (r0 >= r1) return;
@@ -263,40 +266,58 @@ moe_expert_product_mfma_kernel(const uint16_t* __restrict__ a, int a_stride, con
     const uint16_t* w1 = w + (size_t)e * w_expert_stride + (size_t)(c0 + r) * K + 8 * kq;
     const uint16_t* w2 = w1 + (size_t)N * K;
     const int steps = K / 32;
-    for (int rb = r0; rb < r1; rb += 16) {
-        const int row = rb + r;
-        const bool row_ok = row < r1;
-        const uint16_t* ar = a + (size_t)(row_ok ? row : r1 - 1) * a_stride + 8 * kq;
-        moe_v4f acc = moe_v4f{0.f, 0.f, 0.f, 0.f}, acc2 = acc;
-#pragma unroll 4
+    for (int rb = r0; rb < r1; rb += 16 * MT) {
+        const bool two = rb + 16 < r1;                    // the same for the whole block
+        const uint16_t* ar[MT];
+        bool row_ok[MT];
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+            const int row = rb + 16 * m + r;
+            row_ok[m] = row < r1;
+            ar[m] = a + (size_t)(row_ok[m] ? row : r1 - 1) * a_stride + 8 * kq;
+        }
+        moe_v4f acc[MT][NW];
+#pragma unroll
+        for (int m = 0; m < MT; ++m)
+#pragma unroll
+            for (int n = 0; n < NW; ++n) acc[m][n] = moe_v4f{0.f, 0.f, 0.f, 0.f};
         for (int s = wave; s < steps; s += 4) {
-            const uint4 wa = load_stream16(w1 + 32 * s);
-            uint4 xa = *reinterpret_cast<const uint4*>(ar + 32 * s);
-            if (!row_ok) xa = uint4{0u, 0u, 0u, 0u};
-            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(moe_v8b, wa), __builtin_bit_cast(moe_v8b, xa), acc, 0, 0, 0);
-            if (GLU) {
-                const uint4 wb = load_stream16(w2 + 32 * s);
-                acc2 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(moe_v8b, wb), __builtin_bit_cast(moe_v8b, xa), acc2, 0, 0, 0);
+            uint4 wv[NW];
+            wv[0] = load_stream16(w1 + 32 * s);
+            if (GLU) wv[NW - 1] = load_stream16(w2 + 32 * s);
+#pragma unroll
+            for (int m = 0; m < MT; ++m) {
+                if (m == 0 || two) {
+                    uint4 xa = *reinterpret_cast<const uint4*>(ar[m] + 32 * s);
+                    if (!row_ok[m]) xa = uint4{0u, 0u, 0u, 0u};
+#pragma unroll
+                    for (int n = 0; n < NW; ++n)
+                        acc[m][n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(moe_v8b, wv[n]), __builtin_bit_cast(moe_v8b, xa),
+                                                                           acc[m][n], 0, 0, 0);
+                }
             }
         }
-        __syncthreads();                                   // the chunk before has been summed
+        __syncthreads();                                   // the pass before has been summed
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            sums[wave][0][4 * kq + i][r] = acc[i];
-            if (GLU) sums[wave][GLU ? 1 : 0][4 * kq + i][r] = acc2[i];
-        }
+        for (int m = 0; m < MT; ++m)
+#pragma unroll
+            for (int n = 0; n < NW; ++n)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) sums[wave][m][n][4 * kq + i][r] = acc[m][n][i];
         __syncthreads();
-        {
-            const int col = tid >> 4, j = tid & 15;        // 256 threads: 16 columns x 16 token rows
-            if (rb + j < r1) {
-                float v = sums[0][0][col][j] + sums[1][0][col][j] + sums[2][0][col][j] + sums[3][0][col][j];
+        const int col = tid >> 4, j = tid & 15;            // 256 threads: 16 columns x 16 token rows
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+            const int row = rb + 16 * m + j;
+            if (row < r1) {
+                float v = sums[0][m][0][col][j] + sums[1][m][0][col][j] + sums[2][m][0][col][j] + sums[3][m][0][col][j];
                 if (GLU) {
-                    const float u2 = sums[0][GLU ? 1 : 0][col][j] + sums[1][GLU ? 1 : 0][col][j] + sums[2][GLU ? 1 : 0][col][j] + sums[3][GLU ? 1 : 0][col][j];
+                    const float u2 = sums[0][m][NW - 1][col][j] + sums[1][m][NW - 1][col][j] + sums[2][m][NW - 1][col][j] + sums[3][m][NW - 1][col][j];
                     // gate and up are rounded to bfloat16 first, as a product kernel followed by the gated unit's kernel leaves them
                     const float g = bf16_bits_to_f32(f32_to_bf16_bits(v)), u = bf16_bits_to_f32(f32_to_bf16_bits(u2));
                     v = u * (g / (1.0f + expf(-g)));
                 }
-                out[(size_t)(rb + j) * out_stride + c0 + col] = f32_to_bf16_bits(v);
+                out[(size_t)row * out_stride + c0 + col] = f32_to_bf16_bits(v);
             }
         }
     }
