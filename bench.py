@@ -234,7 +234,7 @@ def _design_configs(z, layers):
     # between eight experts of a quarter of that size, two per token, beside a shared one of the same size; a gate on every
     # sublayer's result and a token input of 64 columns per layer
     fiz_att = dict(heads=z["heads"], kv_heads=z["kv"], dim=z["dim"], vdim=z["vdim"], scale=z["dim"] ** -0.5,
-                   mask=dict(size=z["window"], pool=64), rot=dict(base=250000.0, dims=z["dim"] // 2))
+                   mask=dict(size=z["window"], pool=64), rot=dict(base=500000.0, dims=z["dim"] // 2))
     fiz_moe = dict(kind="moe", router=dict(experts=8, top=2), expert=dict(ff=z["ff"] // 4), shared=dict(ff=z["ff"] // 4))
     fiz_kinds = [("attention", fiz_att, dict(kind="dense", ff=z["ff"])), ("mamba2", ssm, fiz_moe), ("attention", fiz_att, fiz_moe),
                  ("mamba2", ssm, dict(kind="dense", ff=z["ff"]))]

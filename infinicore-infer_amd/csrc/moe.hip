@@ -375,33 +375,39 @@ IC_EXPORT int ic_moe_expert_product(const void* a, int a_stride, const void* w, 
 }
 
 // ---------------------------------------------------------------------------------------------
-// out[t] = sum_k y[place[t * top + k]] * (weights[t * top + k] or 1) + shared[t].  grid (T).
+// out[t] = sum_k y[place[t * top + k]] * (weights[t * top + k] or 1) + shared[t].  grid (T, ceil(d / 256)), a thread a column:
+// the pairs' places are read once, then the top + 1 loads of a column are in flight together.
 // ---------------------------------------------------------------------------------------------
 template <typename T>
 __global__ void __launch_bounds__(256)
 moe_combine_kernel(const T* __restrict__ y, int y_stride, const int* __restrict__ place, const float* __restrict__ weights,
                    const T* __restrict__ shared, int shared_stride, int top, int d, T* __restrict__ out, int out_stride) {
-    const int t = blockIdx.x;
-    for (int i = threadIdx.x; i < d; i += blockDim.x) {
-        float s = shared ? to_f32(shared[(size_t)t * shared_stride + i]) : 0.f;
-        for (int k = 0; k < top; ++k) {
-            const int pair = t * top + k;
-            s += to_f32(y[(size_t)place[pair] * y_stride + i]) * (weights ? weights[pair] : 1.f);
-        }
-        out[(size_t)t * out_stride + i] = from_f32<T>(s);
+    const int t = blockIdx.x, i = blockIdx.y * 256 + threadIdx.x;
+    if (i >= d) return;
+    int at[kMoeMaxTop];
+    float wt[kMoeMaxTop];
+#pragma unroll
+    for (int k = 0; k < kMoeMaxTop; ++k) {
+        at[k] = k < top ? place[t * top + k] : 0;
+        wt[k] = (k < top && weights) ? weights[t * top + k] : 1.f;
     }
+    float s = shared ? to_f32(shared[(size_t)t * shared_stride + i]) : 0.f;
+#pragma unroll
+    for (int k = 0; k < kMoeMaxTop; ++k)
+        if (k < top) s += to_f32(y[(size_t)at[k] * y_stride + i]) * wt[k];
+    out[(size_t)t * out_stride + i] = from_f32<T>(s);
 }
 
 IC_EXPORT int ic_moe_combine(const void* y, int y_stride, int dtype, const int* place, const float* weights,
                              const void* shared, int shared_stride, int T, int top, int d, void* out, int out_stride,
                              hipStream_t stream) {
     if (T <= 0) return IC_OK;
-    if (top <= 0 || d <= 0) return IC_ERR_ARG;
+    if (top <= 0 || top > kMoeMaxTop || d <= 0 || (d + 255) / 256 > 65535) return IC_ERR_ARG;
     if (dtype == IC_F32)
-        hipLaunchKernelGGL(moe_combine_kernel<float>, dim3(T), dim3(256), 0, stream, (const float*)y, y_stride, place, weights,
+        hipLaunchKernelGGL(moe_combine_kernel<float>, dim3(T, (d + 255) / 256), dim3(256), 0, stream, (const float*)y, y_stride, place, weights,
                            (const float*)shared, shared_stride, top, d, (float*)out, out_stride);
     else if (dtype == IC_BF16)
-        hipLaunchKernelGGL(moe_combine_kernel<bf16>, dim3(T), dim3(256), 0, stream, (const bf16*)y, y_stride, place, weights,
+        hipLaunchKernelGGL(moe_combine_kernel<bf16>, dim3(T, (d + 255) / 256), dim3(256), 0, stream, (const bf16*)y, y_stride, place, weights,
                            (const bf16*)shared, shared_stride, top, d, (bf16*)out, out_stride);
     else
         return IC_ERR_UNSUPPORTED;

