@@ -268,3 +268,37 @@ def test_the_plain_state_space_recurrence_against_its_closed_form():
     x, w, b = torch.randn(9, 3, generator=g, dtype=torch.float64), torch.randn(3, 4, generator=g, dtype=torch.float64), torch.randn(3, dtype=torch.float64, generator=g)
     pad = torch.cat([torch.zeros(3, 3, dtype=torch.float64), x])
     assert torch.allclose(P.short_conv(x, w, b), b + sum(w[:, k] * pad[k:k + 9] for k in range(4)))
+
+
+def test_the_scheduler_plans_with_rows_per_block_of_tokens():
+    """The scheduler over a cache with a window group and a group of block rows (a stand-in engine on the real cache
+    manager): portions, decoding and preemption by recompute give every request its continuation, the block group's pool
+    is what runs out first, and every page comes back."""
+    from test_scheduler import FakeEngine, _expected, _task
+    from infinicore_infer_amd.engine.scheduler import Scheduler
+
+    class TwoGroups(FakeEngine):
+        def __init__(self, pages, page_size=4, max_requests=4):
+            self.cache = CacheManager([GroupSpec("window", 1, 8, 8, (0,)), GroupSpec("full", 1, 8, None, (0,), stride=2, of_blocks=True)],
+                                      pages, page_size, max_requests, None)
+            self.history, self.steps = {}, []
+
+        def step(self, entries):
+            rows = super().step(entries)
+            for e in entries:
+                self.cache.trim(e.req_id)
+                assert len(self.cache.requests[e.req_id].tables[1]) == self.cache.pages_for_tokens(self.cache.length(e.req_id))[1]
+            return rows
+
+    eng = TwoGroups([64, 9])                       # blocks of two tokens, pages of four rows: a page of the block group per 8 tokens
+    s = Scheduler(eng, max_batch_tokens=24, chunk_size=16)
+    prompts = {i: list(range(i, i + n)) for i, n in enumerate([30, 9, 17])}
+    for i, p in prompts.items():
+        s.add(_task(i, p, 12))
+    while s.has_unfinished():
+        s.step()
+    done = {t.id: t for t in s.finished}
+    for i, p in prompts.items():
+        assert done[i].generated == _expected(p, 12)
+    assert s.n_preempted > 0                       # 42 + 21 + 29 tokens need 6 + 3 + 4 pages of the block group's nine
+    assert eng.cache.free_pages(0) == 64 and eng.cache.free_pages(1) == 9 and not eng.cache.requests
