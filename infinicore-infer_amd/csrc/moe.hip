@@ -64,44 +64,48 @@ IC_EXPORT int ic_moe_route(const float* z, int z_stride, int T, int E, int top, 
 }
 
 // ---------------------------------------------------------------------------------------------
-// Block e (one wave) walks all pairs twice: first it counts those of experts below e (its offset), then it
-// hands its own pairs their places in order of appearance.
+// Block e takes the pairs in 256 contiguous runs, a thread a run: it counts its run's pairs of experts below e and of e
+// itself, the counts meet in LDS (the pairs below e are the expert's offset, the pairs of e in the runs before a thread's
+// are where its own begin), and a second walk over the run hands e's pairs their places in order of appearance.
 // ---------------------------------------------------------------------------------------------
-__global__ void __launch_bounds__(64)
+__global__ void __launch_bounds__(256)
 moe_sort_kernel(const int* __restrict__ ids, int n, int E, int* __restrict__ offsets, int* __restrict__ order,
                 int* __restrict__ place) {
-    const int e = blockIdx.x, lane = threadIdx.x;
+    __shared__ int below_s[256], mine_s[256];
+    const int e = blockIdx.x, tid = threadIdx.x;
+    const int run = (n + 255) / 256;
+    const int lo = min(n, tid * run), hi = min(n, lo + run);
     int below = 0, mine = 0;
-    for (int i = lane; i < n; i += 64) {
+    for (int i = lo; i < hi; ++i) {
         const int id = ids[i];
         below += id < e;
         mine += id == e;
     }
-    for (int o = 32; o > 0; o >>= 1) {
-        below += __shfl_xor(below, o, kWave);
-        mine += __shfl_xor(mine, o, kWave);
+    below_s[tid] = below;
+    mine_s[tid] = mine;
+    __syncthreads();
+    int total_below = 0, before = 0, total_mine = 0;
+    for (int j = 0; j < 256; ++j) {
+        total_below += below_s[j];
+        before += j < tid ? mine_s[j] : 0;
+        total_mine += mine_s[j];
     }
-    if (lane == 0) {
-        offsets[e] = below;
-        if (e == E - 1) offsets[E] = below + mine;
+    if (tid == 0) {
+        offsets[e] = total_below;
+        if (e == E - 1) offsets[E] = total_below + total_mine;
     }
-    int base = below;
-    for (int i0 = 0; i0 < n; i0 += 64) {
-        const int i = i0 + lane;
-        const bool hit = i < n && ids[i] == e;
-        const unsigned long long m = __ballot(hit);
-        if (hit) {
-            const int at = base + __popcll(m & ((1ull << lane) - 1ull));
+    int at = total_below + before;
+    for (int i = lo; i < hi; ++i)
+        if (ids[i] == e) {
             order[at] = i;
             place[i] = at;
+            ++at;
         }
-        base += __popcll(m);
-    }
 }
 
 IC_EXPORT int ic_moe_sort(const int* ids, int n, int E, int* offsets, int* order, int* place, hipStream_t stream) {
     if (E <= 0 || E > kMoeMaxExperts || n < 0) return IC_ERR_ARG;
-    hipLaunchKernelGGL(moe_sort_kernel, dim3(E), dim3(64), 0, stream, ids, n, E, offsets, order, place);
+    hipLaunchKernelGGL(moe_sort_kernel, dim3(E), dim3(256), 0, stream, ids, n, E, offsets, order, place);
     return ic_launch_status();
 }
 
@@ -375,41 +379,72 @@ IC_EXPORT int ic_moe_expert_product(const void* a, int a_stride, const void* w, 
 }
 
 // ---------------------------------------------------------------------------------------------
-// out[t] = sum_k y[place[t * top + k]] * (weights[t * top + k] or 1) + shared[t].  grid (T, ceil(d / 256)), a thread a column:
-// the pairs' places are read once, then the top + 1 loads of a column are in flight together.
+// out[t] = sum_k y[place[t * top + k]] * (weights[t * top + k] or 1) + shared[t].  grid (T, blocks over the columns), a
+// thread 16 bytes of columns (one column where rows are not made of whole 16-byte pieces): the pairs' places are read
+// once, then the top + 1 loads of a piece are in flight together.
 // ---------------------------------------------------------------------------------------------
-template <typename T>
+template <typename T> __device__ __forceinline__ void moe_store(T* p, const float* o);
+template <> __device__ __forceinline__ void moe_store<float>(float* p, const float* o) {
+    *reinterpret_cast<float4*>(p) = make_float4(o[0], o[1], o[2], o[3]);
+}
+template <> __device__ __forceinline__ void moe_store<bf16>(bf16* p, const float* o) {
+    uint4 v;
+    v.x = (uint32_t)f32_to_bf16_bits(o[0]) | ((uint32_t)f32_to_bf16_bits(o[1]) << 16);
+    v.y = (uint32_t)f32_to_bf16_bits(o[2]) | ((uint32_t)f32_to_bf16_bits(o[3]) << 16);
+    v.z = (uint32_t)f32_to_bf16_bits(o[4]) | ((uint32_t)f32_to_bf16_bits(o[5]) << 16);
+    v.w = (uint32_t)f32_to_bf16_bits(o[6]) | ((uint32_t)f32_to_bf16_bits(o[7]) << 16);
+    *reinterpret_cast<uint4*>(p) = v;
+}
+
+template <typename T, bool VEC>
 __global__ void __launch_bounds__(256)
 moe_combine_kernel(const T* __restrict__ y, int y_stride, const int* __restrict__ place, const float* __restrict__ weights,
                    const T* __restrict__ shared, int shared_stride, int top, int d, T* __restrict__ out, int out_stride) {
-    const int t = blockIdx.x, i = blockIdx.y * 256 + threadIdx.x;
+    constexpr int V = VEC ? MoeVec<T>::N : 1;
+    const int t = blockIdx.x, i = (blockIdx.y * 256 + threadIdx.x) * V;
     if (i >= d) return;
-    int at[kMoeMaxTop];
-    float wt[kMoeMaxTop];
+    float s[V];
+    if (VEC) {
+        if (shared) MoeVec<T>::load(shared + (size_t)t * shared_stride + i, s);
+        else
 #pragma unroll
-    for (int k = 0; k < kMoeMaxTop; ++k) {
-        at[k] = k < top ? place[t * top + k] : 0;
-        wt[k] = (k < top && weights) ? weights[t * top + k] : 1.f;
+            for (int j = 0; j < V; ++j) s[j] = 0.f;
+    } else {
+        s[0] = shared ? to_f32(shared[(size_t)t * shared_stride + i]) : 0.f;
     }
-    float s = shared ? to_f32(shared[(size_t)t * shared_stride + i]) : 0.f;
+    for (int k = 0; k < top; ++k) {
+        const int pair = t * top + k;
+        const float w = weights ? weights[pair] : 1.f;
+        const T* row = y + (size_t)place[pair] * y_stride + i;
+        if (VEC) {
+            float v[V];
+            MoeVec<T>::load(row, v);
 #pragma unroll
-    for (int k = 0; k < kMoeMaxTop; ++k)
-        if (k < top) s += to_f32(y[(size_t)at[k] * y_stride + i]) * wt[k];
-    out[(size_t)t * out_stride + i] = from_f32<T>(s);
+            for (int j = 0; j < V; ++j) s[j] += v[j] * w;
+        } else {
+            s[0] += to_f32(row[0]) * w;
+        }
+    }
+    if (VEC) moe_store<T>(out + (size_t)t * out_stride + i, s);
+    else out[(size_t)t * out_stride + i] = from_f32<T>(s[0]);
 }
 
 IC_EXPORT int ic_moe_combine(const void* y, int y_stride, int dtype, const int* place, const float* weights,
                              const void* shared, int shared_stride, int T, int top, int d, void* out, int out_stride,
                              hipStream_t stream) {
     if (T <= 0) return IC_OK;
-    if (top <= 0 || top > kMoeMaxTop || d <= 0 || (d + 255) / 256 > 65535) return IC_ERR_ARG;
-    if (dtype == IC_F32)
-        hipLaunchKernelGGL(moe_combine_kernel<float>, dim3(T, (d + 255) / 256), dim3(256), 0, stream, (const float*)y, y_stride, place, weights,
-                           (const float*)shared, shared_stride, top, d, (float*)out, out_stride);
-    else if (dtype == IC_BF16)
-        hipLaunchKernelGGL(moe_combine_kernel<bf16>, dim3(T, (d + 255) / 256), dim3(256), 0, stream, (const bf16*)y, y_stride, place, weights,
-                           (const bf16*)shared, shared_stride, top, d, (bf16*)out, out_stride);
-    else
-        return IC_ERR_UNSUPPORTED;
+    if (top <= 0 || top > kMoeMaxTop || d <= 0 || (dtype != IC_F32 && dtype != IC_BF16)) return IC_ERR_ARG;
+    const int V = dtype == IC_F32 ? 4 : 8;
+    const bool vec = d % V == 0 && y_stride % V == 0 && out_stride % V == 0 && (!shared || shared_stride % V == 0) &&
+                     ((uintptr_t)y % 16) == 0 && ((uintptr_t)out % 16) == 0 && ((uintptr_t)shared % 16) == 0;
+    const int per = 256 * (vec ? V : 1);
+    dim3 grid((unsigned)T, (unsigned)((d + per - 1) / per)), block(256);
+    if (grid.y > 65535) return IC_ERR_ARG;
+#define IC_MC(TT, VV)                                                                                                   \
+    hipLaunchKernelGGL((moe_combine_kernel<TT, VV>), grid, block, 0, stream, (const TT*)y, y_stride, place, weights,      \
+                       (const TT*)shared, shared_stride, top, d, (TT*)out, out_stride)
+    if (dtype == IC_F32) { if (vec) IC_MC(float, true); else IC_MC(float, false); }
+    else { if (vec) IC_MC(bf16, true); else IC_MC(bf16, false); }
+#undef IC_MC
     return ic_launch_status();
 }
