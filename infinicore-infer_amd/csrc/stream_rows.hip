@@ -493,6 +493,15 @@ IC_EXPORT int ic_activation(const void* in, void* out, int dtype, long long n, i
 // g null: no gate (the kernel is then the plain norm into the stream).  One block per row.
 // ---------------------------------------------------------------------------------------------
 constexpr int kGnKeep = 16;       // gated values a thread keeps between the two passes (rows up to 256 * 16 wide)
+constexpr int kGnPieces = 4;      // the same in 16-byte pieces of the row (rows up to 256 * 4 pieces wide)
+
+// sigmoid for a gate: float32 rows divide and call expf; rows that are rounded to bfloat16 take the hardware's exp2 and
+// reciprocal (each good to an ulp)
+template <typename T> __device__ __forceinline__ float gate_sigmoid(float z);
+template <> __device__ __forceinline__ float gate_sigmoid<float>(float z) { return 1.0f / (1.0f + expf(-z)); }
+template <> __device__ __forceinline__ float gate_sigmoid<bf16>(float z) {
+    return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * z));
+}
 
 template <typename TY, typename TC>
 __global__ void __launch_bounds__(256)
@@ -504,7 +513,7 @@ gated_norm_into_stream_kernel(const TY* __restrict__ y, const TY* __restrict__ g
     const TY* gr = g ? g + (size_t)t * g_stride : nullptr;
     auto gated = [&](int i) {
         float v = to_f32(yr[i]);
-        if (gr) v *= 1.0f / (1.0f + expf(-(to_f32(gr[i]) + (gb ? gb[i] : 0.f))));
+        if (gr) v *= gate_sigmoid<TY>(to_f32(gr[i]) + (gb ? gb[i] : 0.f));
         return v;
     };
     float keep[kGnKeep];
@@ -538,12 +547,86 @@ gated_norm_into_stream_kernel(const TY* __restrict__ y, const TY* __restrict__ g
     }
 }
 
+// The same for rows made of whole 16-byte pieces (d, the gate's stride and every address a multiple of a piece): a thread
+// a piece, every access 16 bytes.
+template <typename TY>
+__global__ void __launch_bounds__(256)
+gated_norm_into_stream_vec_kernel(const TY* __restrict__ y, const TY* __restrict__ g, int g_stride, const float* __restrict__ gb,
+                                  const float* __restrict__ w, float* __restrict__ x, TY* __restrict__ copy, int d, float eps) {
+    constexpr int N = RowPack<TY>::N;
+    __shared__ float red[16];
+    const int t = blockIdx.x, pieces = d / N;
+    const TY* yr = y + (size_t)t * d;
+    const TY* gr = g ? g + (size_t)t * g_stride : nullptr;
+    auto gated = [&](int c, float* v) {
+        RowPack<TY>::load(yr + c * N, v);
+        if (gr) {
+            float z[N], bz[N];
+            RowPack<TY>::load(gr + c * N, z);
+            if (gb) load_floats<N>(gb + c * N, bz);
+#pragma unroll
+            for (int j = 0; j < N; ++j) v[j] *= gate_sigmoid<TY>(z[j] + (gb ? bz[j] : 0.f));
+        }
+    };
+    float keep[kGnPieces][N];
+    float ss = 0.f;
+#pragma unroll
+    for (int n = 0; n < kGnPieces; ++n) {
+        const int c = threadIdx.x + n * 256;
+        if (c < pieces) {
+            gated(c, keep[n]);
+#pragma unroll
+            for (int j = 0; j < N; ++j) ss += keep[n][j] * keep[n][j];
+        }
+    }
+    for (int c = threadIdx.x + kGnPieces * 256; c < pieces; c += 256) {
+        float v[N];
+        gated(c, v);
+#pragma unroll
+        for (int j = 0; j < N; ++j) ss += v[j] * v[j];
+    }
+    ss = block_sum(ss, red);
+    const float r = 1.0f / sqrtf(ss / (float)d + eps);
+    float* xr = x + (size_t)t * d;
+    auto into = [&](int c, const float* v) {
+        float xs[N], ws[N];
+        load_floats<N>(xr + c * N, xs);
+        load_floats<N>(w + c * N, ws);
+#pragma unroll
+        for (int j = 0; j < N; ++j) xs[j] += v[j] * r * ws[j];
+#pragma unroll
+        for (int j = 0; j < N / 4; ++j)
+            *reinterpret_cast<float4*>(xr + c * N + 4 * j) = make_float4(xs[4 * j], xs[4 * j + 1], xs[4 * j + 2], xs[4 * j + 3]);
+        if (copy) RowPack<TY>::store(copy + (size_t)t * d + c * N, xs);
+    };
+#pragma unroll
+    for (int n = 0; n < kGnPieces; ++n) {
+        const int c = threadIdx.x + n * 256;
+        if (c < pieces) into(c, keep[n]);
+    }
+    for (int c = threadIdx.x + kGnPieces * 256; c < pieces; c += 256) {
+        float v[N];
+        gated(c, v);
+        into(c, v);
+    }
+}
+
 IC_EXPORT int ic_gated_norm_into_stream(const void* y, const void* g, int g_stride, int y_dtype, const float* gb, const float* w,
                                         float* x, void* copy, int copy_dtype, int T, int d, float eps, hipStream_t stream) {
     if (T <= 0) return IC_OK;
     if (d <= 0) return IC_ERR_ARG;
     dim3 grid(T), block(256);
-    if (y_dtype == IC_F32 && (copy == nullptr || copy_dtype == IC_F32))
+    const int piece = y_dtype == IC_BF16 ? 8 : 4;
+    const auto aligned = [](const void* p) { return ((uintptr_t)p % 16) == 0; };
+    const bool vec = d % piece == 0 && (g == nullptr || g_stride % piece == 0) && aligned(y) && aligned(g) && aligned(gb) && aligned(w) &&
+                     aligned(x) && aligned(copy) && (copy == nullptr || copy_dtype == y_dtype);
+    if (vec && y_dtype == IC_F32)
+        hipLaunchKernelGGL(gated_norm_into_stream_vec_kernel<float>, grid, block, 0, stream, (const float*)y, (const float*)g, g_stride,
+                           gb, w, x, (float*)copy, d, eps);
+    else if (vec && y_dtype == IC_BF16)
+        hipLaunchKernelGGL(gated_norm_into_stream_vec_kernel<bf16>, grid, block, 0, stream, (const bf16*)y, (const bf16*)g, g_stride,
+                           gb, w, x, (bf16*)copy, d, eps);
+    else if (y_dtype == IC_F32 && (copy == nullptr || copy_dtype == IC_F32))
         hipLaunchKernelGGL((gated_norm_into_stream_kernel<float, float>), grid, block, 0, stream, (const float*)y, (const float*)g,
                            g_stride, gb, w, x, (float*)copy, d, eps);
     else if (y_dtype == IC_BF16 && (copy == nullptr || copy_dtype == IC_BF16))

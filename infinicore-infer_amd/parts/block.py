@@ -251,8 +251,8 @@ class SandwichGatedBlock(Block):
         self.gated = bool(gated)
         self.side = dict(side) if side else None
         self.side_norm = build_part("norm", self.side["norm"], runtime) if self.side else None
-        if self.side_norm is not None and not hasattr(self.side_norm, "forward_into_stream"):
-            raise ValueError("block %s: norm part %s cannot normalise into the stream" % (name, type(self.side_norm).__name__))
+        if self.side_norm is not None and self.side_norm.deferred() is None:
+            raise ValueError("block %s: norm part %s is not a weighted RMS norm" % (name, type(self.side_norm).__name__))
         self.gates = {}
         self.side_gate = self.side_proj = self.side_table = None
 
@@ -325,5 +325,6 @@ class SandwichGatedBlock(Block):
             ops.token_gate(z, self.side_table, ctx.tokens, s["first_column"], g)
             y = ctx.ws.buffer("side_y", tuple(x.shape), rt.dtype)
             linear(g, self.side_proj, y, rt.gemm_impl, ws=ctx.ws)
-            self.side_norm.forward_into_stream(y, x)
+            weight, eps = self.side_norm.deferred()
+            ops.gated_norm_into_stream(y, None, None, weight, x, eps)          # no gate: the plain norm into the stream
         return None
