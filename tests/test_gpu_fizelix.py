@@ -495,6 +495,8 @@ ATTENTION_CASES = [
     (3, 1, 24, 40, 17, 20, 16),
     (2, 1, 16, 16, 1, 1, 16),
     (2, 2, 32, 32, 48, 0, 16),
+    (6, 2, 64, 128, 20, 4, 16),            # three query heads a kv head; (10, 2, ..): five, two walks of the single tokens' kernel
+    (10, 2, 128, 64, 70, 7, 32),
 ]
 
 
@@ -513,7 +515,7 @@ def test_attention_over_a_window_and_block_means(case, dname, dtype, tol):
     g = torch.Generator().manual_seed(7)
     kc, vc, bt = pg.kc.cuda(), pg.vc.cuda(), pg.bt.cuda()
     kp, vp, pt = (pg.kp.cuda(), pg.vp.cuda(), pg.pt.cuda()) if block else (None, None, None)
-    bias = torch.tensor(([-2.0, 0.5, -4.0, 1.0] * 2)[:H_])
+    bias = torch.tensor(([-2.0, 0.5, -4.0, 1.0] * 3)[:H_])
 
     def run(kernel, req_rows):
         qs, refs, token_req, positions, tiles, row = [], [], [], [], [], 0
